@@ -1114,6 +1114,89 @@ int vmx_gupuvik_forward(vmx_gupuvik *m, const int32_t *tokens, const int32_t *po
                         const int32_t *state_slots, const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids,
                         float *layer_trace, void *stream);
 
+/* ------------------------------------------------- query/key preparation, score extras, gated recurrence, Vokepel executor */
+
+/* A step's projected rows made ready for vmx_window_attention_ex, one launch: q_out[t] = q[t] and the key row, each optionally
+ * RMS-normed over the WHOLE row (x / sqrt(mean(x^2) + eps) * w with bf16 gains of q_width / k_width numbers; NULL: no norm), then
+ * optionally rotated: inside every head of head_dim numbers, coordinates (2i, 2i + 1) with 2i < rot_dims turn by the angle
+ * positions[t] * inv_freq[i] (f32 table of rot_dims / 2 numbers; NULL or rot_dims 0: no rotation).  The key row goes to cache
+ * row slots[t] of k_cache, the value row v[t] AS IT IS to v_cache (v may be the raw key rows: values = keys before the norm);
+ * negative slot: not stored.  q_out [tokens, q_width] f32 must not alias q. */
+int vmx_qk_prepare_cache_write(float *q_out, const float *q, int64_t ldq, int q_width, const float *k, int64_t ldk, int k_width,
+                               const float *v, int64_t ldv, int v_width, const uint16_t *q_norm_bf16, const uint16_t *k_norm_bf16,
+                               float eps, const float *inv_freq, int rot_dims, int head_dim, const int32_t *positions,
+                               const int32_t *slots, void *k_cache, void *v_cache, int cache_dtype, int tokens, void *stream);
+
+/* What vmx_window_attention_ex adds to vmx_window_attention's score shaping; every pointer may be NULL (= not there). */
+typedef struct vmx_window_attn_extras {
+    const uint16_t *sink_bf16;      /* [heads]: the softmax denominator also holds exp(sink[h]): no key, no value, not scaled, once */
+    const uint16_t *dist_r1_bf16;   /* [heads], with dist_r2_bf16 [heads]: score -= r1[h] * ln(1 + r2[h] * (i - j)), after the soft cap */
+    const uint16_t *dist_r2_bf16;
+    const uint16_t *talk_bf16;      /* [heads, heads]: score_h <- sum_g talk[h, g] score_g over the visible keys, before the softmax */
+    int gate_per_element;           /* the gate rows hold heads * vdim numbers (one per output element) instead of one per head */
+} vmx_window_attn_extras;
+/* vmx_window_attention with these extras (NULL: none).  Order: scale and temperature, soft cap, distance penalty, mixing of the
+ * heads, mask, softmax (with sink), weighted sum, gate.  Mixing needs heads <= 64 and heads * dim <= 8192. */
+int vmx_window_attention_ex(void *out, int out_dtype, const float *q, int64_t ldq, const void *k_cache, const void *v_cache, int cache_dtype,
+                            const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids, const int32_t *positions,
+                            const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale, float softcap, int window,
+                            int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim, int block_size, const int32_t *seq_starts,
+                            int num_seqs, void *workspace, size_t workspace_bytes, const vmx_window_attn_extras *extras, void *stream);
+
+/* Minimal gated recurrent unit, element by element over `width` channels with carried state:
+ *   z = sigmoid(zl[t]);  c = u[t] + 1/2 where u[t] >= 0, sigmoid(u[t]) below;  S <- (1 - z) S + z c;  y[t] = S * silu(g[t]) (g NULL: S)
+ * zl, u, g are f32 rows (biases already added) at strides ldz / ldu / ldg; y [tokens, width] f32 or bf16.  S lives in
+ * state[state_slots[seq]] ([slots, width] f32); a sequence whose step starts at position 0 starts from zeros.  Tokens are packed:
+ * sequence s owns rows seq_starts[s] .. seq_starts[s + 1] - 1 at consecutive positions.  Everything in f32. */
+size_t vmx_min_gru_state_bytes(int slots, int width);
+int vmx_min_gru(void *y, int y_dtype, const float *zl, int64_t ldz, const float *u, int64_t ldu, const float *g, int64_t ldg, float *state,
+                const int32_t *positions, const int32_t *seq_starts, const int32_t *state_slots, int num_seqs, int tokens, int width,
+                void *stream);
+
+#define VMX_MIXER_TALKING_ATTENTION 3   /* values = raw keys, whole-row q / k norms, distance penalty, mixed heads, element-wise gate */
+#define VMX_MIXER_ATTENTION_GRU 4       /* rotated sink attention and a minimal gated recurrent unit side by side */
+#define VMX_MLP_DENSE_RELU2 4
+
+/* One layer of a Vokepel model: x += m * mixer(norm1(x)); x += m * ff(norm2(x)) (ff may be absent). */
+typedef struct vmx_vokepel_layer_config {
+    int mixer;                  /* VMX_MIXER_TALKING_ATTENTION or VMX_MIXER_ATTENTION_GRU */
+    int heads, kv_heads, dim, vdim;   /* of the (left) attention; the talking attention's values are its keys: vdim = dim */
+    int window;                 /* 0: every earlier key */
+    float scale, softcap;       /* score scale; soft cap of the talking attention (0: none) */
+    int rot_dims;               /* rotated coordinates per head of the sink attention (0: none) */
+    double rot_base;
+    int gru_width;              /* channels of the recurrent unit */
+    float left_scale, right_scale;   /* mixer = left_scale * attention + right_scale * recurrent unit */
+    int mlp;                    /* VMX_MLP_NONE or VMX_MLP_DENSE_RELU2 */
+    int ff;
+} vmx_vokepel_layer_config;
+
+typedef struct vmx_vokepel_config {
+    int vocab, width, num_layers;
+    float norm_eps, residual_mult, logit_scale, logit_softcap;   /* logit_softcap 0: none */
+    int loop_start, loop_stop, loop_times;   /* layers loop_start .. loop_stop - 1 run loop_times times in a row; loop_times 0: no loop */
+    int dtype;                  /* VMX_BF16: bf16 operands and cache; VMX_F32: everything in f32 */
+    int block_size, num_blocks; /* paged key/value cache: rows per block, blocks per layer run */
+    int max_tokens, max_seqs;   /* most tokens / sequences of one forward call */
+    int state_slots;            /* recurrent-state slots (one per live sequence) */
+} vmx_vokepel_config;
+
+typedef struct vmx_vokepel vmx_vokepel;
+int vmx_vokepel_create(const vmx_vokepel_config *cfg, const vmx_vokepel_layer_config *layers, vmx_vokepel **out);
+void vmx_vokepel_destroy(vmx_vokepel *m);
+int vmx_vokepel_num_layer_runs(const vmx_vokepel *m);   /* layers counted as often as they run */
+/* One checkpoint tensor under its name in the file: "embed", "final.norm", "loop.in", "loop.step", "l<i>.norm1|norm2",
+ * "l<i>.mlp.up|down"; talking attention "l<i>.mix.q|k|g|o|q.norm|k.norm|r1|r2|talk"; attention + recurrent unit
+ * "l<i>.mix.left.q|k|v|o|sink", "l<i>.mix.right.z|x|g|o|z.b|x.b": bf16, matrices [out, in]; host or device memory. */
+int vmx_vokepel_load_tensor(vmx_vokepel *m, const char *name, const void *data, size_t bytes, void *stream);
+int vmx_vokepel_missing_tensors(const vmx_vokepel *m);
+/* One step over packed tokens, arguments as vmx_gupuvik_forward.  Every run of a looped layer has a cache and state of its own.
+ * layer_trace (optional): f32 [layer runs, tokens, width], the residual stream after every layer run. */
+int vmx_vokepel_forward(vmx_vokepel *m, const int32_t *tokens, const int32_t *positions, const int32_t *slots, const int32_t *seq_ids,
+                        int num_tokens, const int32_t *block_tables, int num_seqs, int max_blocks_per_seq, const int32_t *seq_starts,
+                        const int32_t *state_slots, const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids,
+                        float *layer_trace, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

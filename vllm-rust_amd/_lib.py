@@ -236,6 +236,16 @@ _SIGS = {
     "vmx_gupuvik_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
     "vmx_gupuvik_missing_tensors": (_i, [_p]),
     "vmx_gupuvik_forward": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _p, _p, _i, _p, _p, _p, _p]),
+    "vmx_qk_prepare_cache_write": (_i, [_p, _p, _i64, _i, _p, _i64, _i, _p, _i64, _i, _p, _p, _f, _p, _i, _i, _p, _p, _p, _p, _i, _i, _p]),
+    "vmx_window_attention_ex": (_i, [_p, _i, _p, _i64, _p, _p, _i, _p, _i, _p, _p, _p, _p, _i64, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _sz, _p, _p]),
+    "vmx_min_gru_state_bytes": (_sz, [_i, _i]),
+    "vmx_min_gru": (_i, [_p, _i, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _i, _i, _i, _p]),
+    "vmx_vokepel_create": (_i, [_p, _p, _p]),
+    "vmx_vokepel_destroy": (None, [_p]),
+    "vmx_vokepel_num_layer_runs": (_i, [_p]),
+    "vmx_vokepel_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
+    "vmx_vokepel_missing_tensors": (_i, [_p]),
+    "vmx_vokepel_forward": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _p, _p, _i, _p, _p, _p, _p]),
 }
 
 
@@ -299,6 +309,28 @@ class GupuvikConfig(C.Structure):
     _fields_ = [
         ("vocab", _i), ("width", _i), ("num_layers", _i), ("norm_eps", _f), ("embed_scale", C.c_double), ("dtype", _i), ("block_size", _i),
         ("num_blocks", _i), ("max_tokens", _i), ("max_seqs", _i), ("state_slots", _i),
+    ]
+
+
+class WindowAttnExtras(C.Structure):
+    """struct vmx_window_attn_extras (include/vmx.h)."""
+    _fields_ = [("sink_bf16", _p), ("dist_r1_bf16", _p), ("dist_r2_bf16", _p), ("talk_bf16", _p), ("gate_per_element", _i)]
+
+
+class VokepelLayerConfig(C.Structure):
+    """struct vmx_vokepel_layer_config (include/vmx.h)."""
+    _fields_ = [
+        ("mixer", _i), ("heads", _i), ("kv_heads", _i), ("dim", _i), ("vdim", _i), ("window", _i), ("scale", _f), ("softcap", _f),
+        ("rot_dims", _i), ("rot_base", C.c_double), ("gru_width", _i), ("left_scale", _f), ("right_scale", _f), ("mlp", _i), ("ff", _i),
+    ]
+
+
+class VokepelConfig(C.Structure):
+    """struct vmx_vokepel_config (include/vmx.h)."""
+    _fields_ = [
+        ("vocab", _i), ("width", _i), ("num_layers", _i), ("norm_eps", _f), ("residual_mult", _f), ("logit_scale", _f), ("logit_softcap", _f),
+        ("loop_start", _i), ("loop_stop", _i), ("loop_times", _i), ("dtype", _i), ("block_size", _i), ("num_blocks", _i), ("max_tokens", _i),
+        ("max_seqs", _i), ("state_slots", _i),
     ]
 
 

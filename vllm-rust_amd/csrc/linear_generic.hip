@@ -32,6 +32,7 @@ __device__ __forceinline__ void linear_store(const VmxLinear &p, int z, int m, i
         const float g = p.aux[(int64_t)m * p.ldaux + n + z * p.aux_bs];
         v *= 1.0f / (1.0f + expf(-g));
     }
+    v *= p.out_scale;
     const int64_t o = (int64_t)m * p.ldc + n + z * p.c_bs;
     if (p.epilogue == VMX_EP_ADD_F32 || p.epilogue == VMX_EP_ADD_MUL_SIGMOID) ((float *)p.C)[o] += v;
     else if (p.c_f32) ((float *)p.C)[o] = v;

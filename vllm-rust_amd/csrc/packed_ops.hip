@@ -141,6 +141,25 @@ __global__ __launch_bounds__(256) void glu_silu_kernel(void *__restrict__ act, i
     else ((uint16_t *)act)[r * ff + j] = vmx_f32_to_bf16(v);
 }
 
+// out[t] = [a[t] | b[t]] (two f32 rows of `width` numbers side by side), in f32 or bf16: the input of a product over both
+__global__ __launch_bounds__(256) void concat2_rows_kernel(void *__restrict__ out, int out_f32, const float *__restrict__ a,
+                                                            const float *__restrict__ b, int width) {
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    if (i >= 2 * width) return;
+    const float v = i < width ? a[(int64_t)t * width + i] : b[(int64_t)t * width + i - width];
+    const int64_t o = (int64_t)t * 2 * width + i;
+    if (out_f32) ((float *)out)[o] = v;
+    else ((uint16_t *)out)[o] = vmx_f32_to_bf16(v);
+}
+
+// x <- cap * tanh(x * scale / cap) (cap 0: x * scale)
+__global__ __launch_bounds__(256) void scale_softcap_kernel(float *__restrict__ x, int64_t n, float scale, float cap) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i] * scale;
+    x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
 }  // namespace
 
 int vmx_embed_scaled_f32(float *x, const uint16_t *embed, const int32_t *tokens, int T, int width, int vocab, float scale, hipStream_t st) {
@@ -188,5 +207,19 @@ int vmx_argmax_f32_rows(int32_t *out, unsigned long long *keys, const float *log
     hipLaunchKernelGGL(argmax_f32_partial_kernel, dim3(chunks, rows), dim3(256), 0, st, keys, logits, vocab, chunks);
     hipLaunchKernelGGL(argmax_f32_final_kernel, dim3(rows), dim3(64), 0, st, out, keys, chunks);
     VMX_CHECK_LAUNCH("argmax");
+    return VMX_OK;
+}
+
+int vmx_concat2_rows(void *out, int out_f32, const float *a, const float *b, int T, int width, hipStream_t st) {
+    if (T <= 0) return VMX_OK;
+    hipLaunchKernelGGL(concat2_rows_kernel, dim3(T, (2 * width + 255) / 256), dim3(256), 0, st, out, out_f32, a, b, width);
+    VMX_CHECK_LAUNCH("concat rows");
+    return VMX_OK;
+}
+
+int vmx_scale_softcap_f32(float *x, int64_t n, float scale, float cap, hipStream_t st) {
+    if (n <= 0) return VMX_OK;
+    hipLaunchKernelGGL(scale_softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, n, scale, cap);
+    VMX_CHECK_LAUNCH("scale + soft cap");
     return VMX_OK;
 }

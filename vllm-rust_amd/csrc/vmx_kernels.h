@@ -199,6 +199,7 @@ struct VmxLinear {
                                        // ADD_MUL_SIGMOID: C += v * sigmoid(aux[m, n]) (f32 C)
     const float *aux = nullptr;
     int64_t ldaux = 0;
+    float out_scale = 1.0f;            // what is stored or added is this times the epilogue's value (C += out_scale * v)
     int exact = 0;                     // 1: multiply in f32 on the vector ALU even where the matrix cores could take bf16 operands
 };
 int vmx_linear_launch(const VmxLinear &p, hipStream_t st);
@@ -240,3 +241,7 @@ int vmx_argmax_f32_rows(int32_t *out, unsigned long long *keys, const float *log
 int vmx_embed_scaled_f32(float *x, const uint16_t *embed, const int32_t *tokens, int T, int width, int vocab, float scale, hipStream_t st);
 // act[r, j] = silu(gu[r, j]) * gu[r, ff + j], gu f32 [rows, 2 ff], act f32 or bf16 [rows, ff]
 int vmx_glu_silu_rows(void *act, int act_f32, const float *gu, int rows, int ff, hipStream_t st);
+// out[t] = [a[t] | b[t]]: two f32 rows of `width` numbers side by side, stored in f32 or bf16
+int vmx_concat2_rows(void *out, int out_f32, const float *a, const float *b, int T, int width, hipStream_t st);
+// x <- cap * tanh(x * scale / cap) over n numbers (cap 0: x * scale)
+int vmx_scale_softcap_f32(float *x, int64_t n, float scale, float cap, hipStream_t st);

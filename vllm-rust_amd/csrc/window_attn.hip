@@ -3,7 +3,11 @@
 // Position i of a sequence sees j <= i when i - j < window (window 0: every earlier key) or j < keep_first (the first tokens of
 // the sequence stay visible after the window has passed them).  No rotation: positions only decide visibility.  Query head h
 // reads key/value head h / (heads / kv_heads); key and value widths may differ.  The head's output may be multiplied by
-// sigmoid(gate[t, h]) (one number per token and head) before it is stored.
+// sigmoid(gate[t, h]) (one number per token and head, or one per output element) before it is stored.
+// Extras (vmx_window_attention_ex), each optional: a learned sink per head in the softmax denominator (exp(sink), no key, no value);
+// a logarithmic distance penalty s_j -= r1[h] * ln(1 + r2[h] * (i - j)) after the soft cap; mixing of the heads' scores,
+// s_h <- sum_g talk[h, g] s_g at every visible key, before the softmax (all heads of a token then run in one workgroup).
+// vmx_qk_prepare_cache_write readies a step's projected rows: whole-row RMS norms of q and k, pair rotation, cache write.
 //
 // Keys and values live in two caches of rows [kv_heads * dim] / [kv_heads * vdim], bf16 or f32; a step writes its new rows first
 // (vmx_kv_cache_write_f32) and prompts, prompt portions and decode tokens then run the SAME kernel over the cache, so a row's
@@ -61,7 +65,76 @@ struct WinAttn {
     int bs_shift;                // log2(block_size) when it is a power of two, else -1
     int parts;                   // > 1: the key tiles of a run are dealt to `parts` workgroups, whose results go to `ws` for the merge
     float *ws;                   // [tokens, heads, parts, vdim + 2]: unnormalised sums, running maximum, denominator
+    const uint16_t *sink, *r1, *r2, *talk;   // extras, each NULL when absent
+    int gate_elem;               // 1: gate rows hold heads * vdim numbers
 };
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// the denominator's sink term: (m, den, f) -> the running maximum with the sink in it, the denominator plus exp(sink - maximum),
+// and the factor the sums gathered under the old maximum take
+__device__ __forceinline__ void add_sink(float sink, float &m, float &den, float &f) {
+    const float mn = fmaxf(m, sink);
+    f = expf(m - mn);
+    den = den * f + expf(sink - mn);
+    m = mn;
+}
+
+// q_out[t] / key row of token t: optional whole-row RMS norm, optional pair rotation inside every head, keys and values to the cache
+__global__ __launch_bounds__(256) void qk_prepare_kernel(float *__restrict__ q_out, const float *__restrict__ q, int64_t ldq, int qw,
+                                                          const float *__restrict__ k, int64_t ldk, int kw, const float *__restrict__ v,
+                                                          int64_t ldv, int vw, const uint16_t *__restrict__ qn, const uint16_t *__restrict__ kn,
+                                                          float eps, const float *__restrict__ inv_freq, int rot_dims, int head_dim,
+                                                          const int32_t *__restrict__ positions, const int32_t *__restrict__ slots,
+                                                          void *__restrict__ kc, void *__restrict__ vc, int f32) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float *qr = q + (int64_t)t * ldq, *kr = k + (int64_t)t * ldk, *vr = v + (int64_t)t * ldv;
+    float qinv = 1.0f, kinv = 1.0f;
+    if (qn) {
+        float ss = 0.f;
+        for (int i = tid; i < qw; i += 256) ss += qr[i] * qr[i];
+        ss = vmx_block_sum_256(ss, red);
+        qinv = 1.0f / sqrtf(ss / (float)qw + eps);
+        __syncthreads();
+    }
+    if (kn) {
+        float ss = 0.f;
+        for (int i = tid; i < kw; i += 256) ss += kr[i] * kr[i];
+        ss = vmx_block_sum_256(ss, red);
+        kinv = 1.0f / sqrtf(ss / (float)kw + eps);
+    }
+    const float pos = (float)positions[t];
+    const int64_t slot = slots[t];
+    const bool rot = inv_freq && rot_dims > 0;
+    for (int i = tid; i < qw + kw; i += 256) {
+        const bool isq = i < qw;
+        const int e = isq ? i : i - qw;
+        const float *src = isq ? qr : kr;
+        const uint16_t *w = isq ? qn : kn;
+        const float inv = isq ? qinv : kinv;
+        float x = src[e] * inv;
+        if (w) x *= vmx_bf16_to_f32(w[e]);
+        const int c = e % head_dim;
+        if (rot && c < rot_dims) {
+            float y = src[e ^ 1] * inv;   // the pair's other coordinate (rot_dims and head_dim are even)
+            if (w) y *= vmx_bf16_to_f32(w[e ^ 1]);
+            float sn, cs;
+            sincosf(pos * inv_freq[c >> 1], &sn, &cs);
+            x = (c & 1) ? x * cs + y * sn : x * cs - y * sn;
+        }
+        if (isq) q_out[(int64_t)t * qw + e] = x;
+        else if (slot >= 0) {
+            if (f32) ((float *)kc)[slot * kw + e] = x;
+            else ((uint16_t *)kc)[slot * kw + e] = vmx_f32_to_bf16(x);
+        }
+    }
+    if (slot >= 0)
+        for (int i = tid; i < vw; i += 256) {
+            if (f32) ((float *)vc)[slot * vw + i] = vr[i];
+            else ((uint16_t *)vc)[slot * vw + i] = vmx_f32_to_bf16(vr[i]);
+        }
+}
 
 constexpr int WA_MAX_DIM = 256;
 
@@ -97,6 +170,7 @@ __global__ __launch_bounds__(256) void window_attn_wave_kernel(const WinAttn p) 
             float d = 0.f;
             for (int i = 0; i < D; i++) d = fmaf(qs[wave][i], ld_cache<F32>(p.kc, kb + i), d);
             s = p.softcap > 0.f ? p.softcap * tanhf(d * inv_cap) : d;
+            if (p.r1) s -= vmx_bf16_to_f32(p.r1[h]) * log1pf(vmx_bf16_to_f32(p.r2[h]) * (float)(pos - j));
         }
         const float mn = fmaxf(m, vmx_wave_max(s));
         const float pj = live ? expf(s - mn) : 0.f;
@@ -117,15 +191,126 @@ __global__ __launch_bounds__(256) void window_attn_wave_kernel(const WinAttn p) 
             }
         }
     }
+    if (p.sink) {
+        float f;
+        add_sink(vmx_bf16_to_f32(p.sink[h]), m, den, f);
+#pragma unroll
+        for (int u = 0; u < VPL; u++) acc[u] *= f;
+    }
     float g = 1.0f / den;
-    if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)t * p.ldgate + h]));
+    if (p.gate && !p.gate_elem) g *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + h]);
 #pragma unroll
     for (int u = 0; u < VPL; u++) {
         const int c = lane + 64 * u;
         if (c < V) {
             const int64_t o = ((int64_t)t * p.heads + h) * V + c;
-            if (p.out_f32) ((float *)p.out)[o] = acc[u] * g;
-            else ((uint16_t *)p.out)[o] = vmx_f32_to_bf16(acc[u] * g);
+            float r = acc[u] * g;
+            if (p.gate && p.gate_elem) r *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + (int64_t)h * V + c]);
+            if (p.out_f32) ((float *)p.out)[o] = r;
+            else ((uint16_t *)p.out)[o] = vmx_f32_to_bf16(r);
+        }
+    }
+}
+
+// The vector form with mixed heads: a workgroup owns ONE token and all its heads (wave w the heads w, w + NW, ...; HPW of them).
+// Per tile of 64 keys every wave leaves the shaped scores of its heads in LDS, then reads all heads' scores of its lane's key and
+// mixes them with its heads' rows of the mixing matrix; softmax and the weighted sum go on per head as in the form above.
+constexpr int TALK_MAX_HEADS = 64, TALK_MAX_QS = 8192;
+template <bool F32, int VPL, int HPW>
+__global__ __launch_bounds__(512) void window_attn_talk_kernel(const WinAttn p) {
+    extern __shared__ float talk_lds[];
+    const int H = p.heads, D = p.dim, V = p.vdim, NW = blockDim.x >> 6;
+    float *qs = talk_lds, *raw = qs + H * D, *tk = raw + H * 64;   // queries [H, D], shaped scores [H, 64], mixing matrix [H, H]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, t = blockIdx.x;
+    const int qpk = H / p.kv_heads;
+    const int64_t kw = (int64_t)p.kv_heads * D, vw = (int64_t)p.kv_heads * V;
+    const int pos = p.positions[t];
+    const int32_t *bt = p.block_tables + (int64_t)p.seq_ids[t] * p.max_blocks;
+    for (int i = threadIdx.x; i < H * D; i += blockDim.x)
+        qs[i] = p.q[(int64_t)t * p.ldq + i] * p.scale * (p.temp ? vmx_bf16_to_f32(p.temp[i / D]) : 1.0f);
+    for (int i = threadIdx.x; i < H * H; i += blockDim.x) tk[i] = vmx_bf16_to_f32(p.talk[i]);
+    __syncthreads();
+    const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    const int na = min(p.keep_first, lo), n = na + (pos - lo + 1);
+    const float inv_cap = p.softcap > 0.f ? 1.0f / p.softcap : 0.f;
+    float m[HPW], den[HPW], acc[HPW][VPL];
+#pragma unroll
+    for (int a = 0; a < HPW; a++) {
+        m[a] = -FLT_MAX, den[a] = 0.f;
+#pragma unroll
+        for (int u = 0; u < VPL; u++) acc[a][u] = 0.f;
+    }
+    for (int base = 0; base < n; base += 64) {
+        const int idx = base + lane;
+        const bool live = idx < n;
+        const int j = idx < na ? idx : lo + (idx - na);
+        const int crow = live ? bt[j / p.block_size] * p.block_size + j % p.block_size : 0;
+#pragma unroll
+        for (int a = 0; a < HPW; a++) {
+            const int h = wave + a * NW;
+            if (h < H && live) {
+                const int64_t kb = (int64_t)crow * kw + (int64_t)(h / qpk) * D;
+                float d = 0.f;
+                for (int i = 0; i < D; i++) d = fmaf(qs[h * D + i], ld_cache<F32>(p.kc, kb + i), d);
+                float sc = p.softcap > 0.f ? p.softcap * tanhf(d * inv_cap) : d;
+                if (p.r1) sc -= vmx_bf16_to_f32(p.r1[h]) * log1pf(vmx_bf16_to_f32(p.r2[h]) * (float)(pos - j));
+                raw[h * 64 + lane] = sc;
+            }
+        }
+        __syncthreads();
+        const int cnt = min(64, n - base);
+#pragma unroll
+        for (int a = 0; a < HPW; a++) {
+            const int h = wave + a * NW;
+            if (h >= H) continue;   // whole waves: no barrier inside
+            float sc = -FLT_MAX;
+            if (live) {
+                sc = 0.f;
+                for (int g = 0; g < H; g++) sc = fmaf(tk[h * H + g], raw[g * 64 + lane], sc);
+            }
+            const float mn = fmaxf(m[a], vmx_wave_max(sc));
+            const float pj = live ? expf(sc - mn) : 0.f;
+            const float f = expf(m[a] - mn);
+            den[a] = den[a] * f + vmx_wave_sum(pj);
+            m[a] = mn;
+#pragma unroll
+            for (int u = 0; u < VPL; u++) acc[a][u] *= f;
+            const int kvh = h / qpk;
+            for (int jj = 0; jj < cnt; jj++) {
+                const float w = __shfl(pj, jj, 64);
+                const int64_t r = __shfl(crow, jj, 64);
+                const int64_t vb = r * vw + (int64_t)kvh * V;
+#pragma unroll
+                for (int u = 0; u < VPL; u++) {
+                    const int c = lane + 64 * u;
+                    if (c < V) acc[a][u] = fmaf(w, ld_cache<F32>(p.vc, vb + c), acc[a][u]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int a = 0; a < HPW; a++) {
+        const int h = wave + a * NW;
+        if (h >= H) continue;
+        if (p.sink) {
+            float f;
+            add_sink(vmx_bf16_to_f32(p.sink[h]), m[a], den[a], f);
+#pragma unroll
+            for (int u = 0; u < VPL; u++) acc[a][u] *= f;
+        }
+        float g = 1.0f / den[a];
+        if (p.gate && !p.gate_elem) g *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + h]);
+#pragma unroll
+        for (int u = 0; u < VPL; u++) {
+            const int c = lane + 64 * u;
+            if (c < V) {
+                const int64_t o = ((int64_t)t * H + h) * V + c;
+                float r = acc[a][u] * g;
+                if (p.gate && p.gate_elem) r *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + (int64_t)h * V + c]);
+                if (p.out_f32) ((float *)p.out)[o] = r;
+                else ((uint16_t *)p.out)[o] = vmx_f32_to_bf16(r);
+            }
         }
     }
 }
@@ -188,6 +373,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
     }
     const float smul = p.scale * (p.temp ? vmx_bf16_to_f32(p.temp[head]) : 1.0f);
     const float inv_cap = p.softcap > 0.f ? 1.0f / p.softcap : 0.f;
+    const float dr1 = p.r1 ? vmx_bf16_to_f32(p.r1[head]) : 0.f, dr2 = p.r1 ? vmx_bf16_to_f32(p.r2[head]) : 0.f;
     // this workgroup's share of the run's key tiles
     const int ntile = (nk + KT - 1) / KT, per = (ntile + p.parts - 1) / p.parts;
     const int kb0 = share * per * KT, kb1 = min(nk, (share + 1) * per * KT);
@@ -271,6 +457,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
                     const bool vis = qlive && idx < kb1 && j <= qi && (p.window == 0 || qi - j < p.window || j < p.keep_first);
                     float x = acc[r] * smul;
                     if (p.softcap > 0.f) x = p.softcap * tanh_fast(x * inv_cap);
+                    if (p.r1) x -= dr1 * __logf(1.0f + dr2 * (float)max(qi - j, 0));
                     sc[kt][r] = vis ? x : -FLT_MAX;
                     tmax = fmaxf(tmax, sc[kt][r]);
                 }
@@ -334,8 +521,16 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
         if (fg == 0) w[V] = m, w[V + 1] = den;
         return;
     }
+    if (p.sink) {
+        float f;
+        add_sink(vmx_bf16_to_f32(p.sink[head]), m, den, f);
+#pragma unroll
+        for (int v = 0; v < VS; v++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[v][r] *= f;
+    }
     float g = 1.0f / den;
-    if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)(r0 + qrow) * p.ldgate + head]));
+    if (p.gate && !p.gate_elem) g *= sigmoid_f32(p.gate[(int64_t)(r0 + qrow) * p.ldgate + head]);
 #pragma unroll
     for (int v = 0; v < VS; v++)
 #pragma unroll
@@ -343,8 +538,10 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
             const int c = 16 * v + 4 * fg + r;
             if (c < V) {
                 const int64_t at = ((int64_t)(r0 + qrow) * p.heads + head) * V + c;
-                if (p.out_f32) ((float *)p.out)[at] = o[v][r] * g;
-                else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(o[v][r] * g);
+                float x = o[v][r] * g;
+                if (p.gate && p.gate_elem) x *= sigmoid_f32(p.gate[(int64_t)(r0 + qrow) * p.ldgate + (int64_t)head * V + c]);
+                if (p.out_f32) ((float *)p.out)[at] = x;
+                else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(x);
             }
         }
 }
@@ -356,10 +553,11 @@ __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) 
     const float *w = p.ws + (int64_t)row * p.parts * (V + 2);
     const bool mine = lane < p.parts;
     const float mq = mine ? w[lane * (V + 2) + V] : -FLT_MAX, dq = mine ? w[lane * (V + 2) + V + 1] : 0.f;
-    const float M = vmx_wave_max(mq);
+    const float sink = p.sink ? vmx_bf16_to_f32(p.sink[h]) : -FLT_MAX;
+    const float M = fmaxf(vmx_wave_max(mq), sink);
     const float eq = mine ? expf(mq - M) : 0.f;            // a share without keys: e^(-huge) = 0
-    float g = 1.0f / vmx_wave_sum(eq * dq);
-    if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)t * p.ldgate + h]));
+    float g = 1.0f / (vmx_wave_sum(eq * dq) + (p.sink ? expf(sink - M) : 0.f));
+    if (p.gate && !p.gate_elem) g *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + h]);
     for (int c0 = 0; c0 < V; c0 += 64) {
         const int c = c0 + lane, cc = min(c, V - 1);
         float x[16];                                       // every share's value first: independent loads, one wait
@@ -370,8 +568,10 @@ __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) 
         for (int q = 0; q < 16; q++) acc = fmaf(__shfl(eq, q, 64), x[q], acc);
         if (c < V) {
             const int64_t at = (int64_t)row * V + c;
-            if (p.out_f32) ((float *)p.out)[at] = acc * g;
-            else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(acc * g);
+            float r = acc * g;
+            if (p.gate && p.gate_elem) r *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + (int64_t)h * V + c]);
+            if (p.out_f32) ((float *)p.out)[at] = r;
+            else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(r);
         }
     }
 }
@@ -395,12 +595,43 @@ extern "C" int vmx_kv_cache_write_f32(const float *k, int64_t ldk, const float *
     return VMX_OK;
 }
 
+extern "C" int vmx_qk_prepare_cache_write(float *q_out, const float *q, int64_t ldq, int q_width, const float *k, int64_t ldk, int k_width,
+                                          const float *v, int64_t ldv, int v_width, const uint16_t *q_norm_bf16, const uint16_t *k_norm_bf16,
+                                          float eps, const float *inv_freq, int rot_dims, int head_dim, const int32_t *positions,
+                                          const int32_t *slots, void *k_cache, void *v_cache, int cache_dtype, int tokens, void *stream) {
+    VMX_REQUIRE(q_out && q && k && v && positions && slots && k_cache && v_cache, "qk_prepare: null pointer");
+    VMX_REQUIRE(q_out != q, "qk_prepare: the prepared queries need rows of their own");
+    VMX_REQUIRE(cache_dtype == VMX_F32 || cache_dtype == VMX_BF16, "qk_prepare: the cache holds f32 or bf16");
+    VMX_REQUIRE(q_width >= 1 && k_width >= 1 && v_width >= 1 && ldq >= q_width && ldk >= k_width && ldv >= v_width, "qk_prepare: bad row widths");
+    VMX_REQUIRE(head_dim >= 1 && q_width % head_dim == 0 && k_width % head_dim == 0, "qk_prepare: rows are not whole heads of %d", head_dim);
+    const bool rot = inv_freq && rot_dims > 0;
+    VMX_REQUIRE(!rot || (rot_dims % 2 == 0 && rot_dims <= head_dim && head_dim % 2 == 0),
+                "qk_prepare: %d rotated coordinates in heads of %d (pairs inside a head of even size)", rot_dims, head_dim);
+    if (tokens <= 0) return VMX_OK;
+    hipLaunchKernelGGL(qk_prepare_kernel, dim3(tokens), dim3(256), 0, vmx_stream(stream), q_out, q, ldq, q_width, k, ldk, k_width, v, ldv, v_width,
+                       q_norm_bf16, k_norm_bf16, eps, inv_freq, rot ? rot_dims : 0, head_dim, positions, slots, k_cache, v_cache,
+                       cache_dtype == VMX_F32);
+    VMX_CHECK_LAUNCH("qk_prepare");
+    return VMX_OK;
+}
+
 extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, int64_t ldq, const void *k_cache, const void *v_cache,
                                     int cache_dtype, const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids,
                                     const int32_t *positions, const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale,
                                     float softcap, int window, int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim,
                                     int block_size, const int32_t *seq_starts, int num_seqs, void *workspace, size_t workspace_bytes,
                                     void *stream) {
+    return vmx_window_attention_ex(out, out_dtype, q, ldq, k_cache, v_cache, cache_dtype, block_tables, max_blocks_per_seq, seq_ids, positions,
+                                   head_temp_bf16, gate, ldgate, scale, softcap, window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size,
+                                   seq_starts, num_seqs, workspace, workspace_bytes, nullptr, stream);
+}
+
+extern "C" int vmx_window_attention_ex(void *out, int out_dtype, const float *q, int64_t ldq, const void *k_cache, const void *v_cache,
+                                       int cache_dtype, const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids,
+                                       const int32_t *positions, const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale,
+                                       float softcap, int window, int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim,
+                                       int block_size, const int32_t *seq_starts, int num_seqs, void *workspace, size_t workspace_bytes,
+                                       const vmx_window_attn_extras *extras, void *stream) {
     VMX_REQUIRE(out && q && k_cache && v_cache && block_tables && seq_ids && positions, "window_attention: null pointer");
     VMX_REQUIRE((out_dtype == VMX_F32 || out_dtype == VMX_BF16) && (cache_dtype == VMX_F32 || cache_dtype == VMX_BF16),
                 "window_attention: f32 or bf16 output and cache");
@@ -408,13 +639,47 @@ extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, in
                 heads, kv_heads);
     VMX_REQUIRE(dim >= 1 && dim <= WA_MAX_DIM && vdim >= 1 && vdim <= 256, "window_attention: head sizes %d / %d outside 1..256", dim, vdim);
     VMX_REQUIRE(window >= 0 && keep_first >= 0 && block_size >= 1 && max_blocks_per_seq >= 1 && softcap >= 0.f, "window_attention: bad arguments");
-    VMX_REQUIRE(ldq >= (int64_t)heads * dim && (!gate || ldgate >= heads), "window_attention: bad row strides");
+    const vmx_window_attn_extras none = {nullptr, nullptr, nullptr, nullptr, 0};
+    const vmx_window_attn_extras &ex = extras ? *extras : none;
+    VMX_REQUIRE(ldq >= (int64_t)heads * dim && (!gate || ldgate >= (ex.gate_per_element ? (int64_t)heads * vdim : heads)),
+                "window_attention: bad row strides");
+    VMX_REQUIRE(!ex.dist_r1_bf16 == !ex.dist_r2_bf16, "window_attention: the distance penalty needs both of its numbers per head");
+    VMX_REQUIRE(!ex.talk_bf16 || (heads <= TALK_MAX_HEADS && heads * dim <= TALK_MAX_QS),
+                "window_attention: mixed heads take at most %d heads and %d query numbers per token", TALK_MAX_HEADS, TALK_MAX_QS);
     if (tokens <= 0) return VMX_OK;
     WinAttn p{out, out_dtype == VMX_F32, q, ldq, k_cache, v_cache, block_tables, seq_ids, positions, max_blocks_per_seq, head_temp_bf16,
               gate, ldgate, scale, softcap, window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size, seq_starts, num_seqs,
-              (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1, 1, (float *)workspace};
+              (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1, 1, (float *)workspace,
+              ex.sink_bf16, ex.dist_r1_bf16, ex.dist_r2_bf16, ex.talk_bf16, ex.gate_per_element ? 1 : 0};
     hipStream_t st = vmx_stream(stream);
     const bool f32 = cache_dtype == VMX_F32;
+    if (p.talk) {   // all heads of a token in one workgroup
+        const int nw = heads < 8 ? heads : 8, hpw = (heads + nw - 1) / nw;
+        const int vpl = vdim <= 64 ? 1 : (vdim <= 128 ? 2 : 4);
+        const size_t lds = ((size_t)heads * dim + (size_t)heads * 64 + (size_t)heads * heads) * 4;
+        const dim3 grid(tokens), block(64 * nw);
+#define WT_LAUNCH(F, U, HP) hipLaunchKernelGGL((window_attn_talk_kernel<F, U, HP>), grid, block, lds, st, p)
+#define WT_HP(F, U)                         \
+    do {                                    \
+        if (hpw == 1) WT_LAUNCH(F, U, 1);   \
+        else if (hpw == 2) WT_LAUNCH(F, U, 2); \
+        else if (hpw <= 4) WT_LAUNCH(F, U, 4); \
+        else WT_LAUNCH(F, U, 8);            \
+    } while (0)
+        if (f32) {
+            if (vpl == 1) WT_HP(true, 1);
+            else if (vpl == 2) WT_HP(true, 2);
+            else WT_HP(true, 4);
+        } else {
+            if (vpl == 1) WT_HP(false, 1);
+            else if (vpl == 2) WT_HP(false, 2);
+            else WT_HP(false, 4);
+        }
+#undef WT_HP
+#undef WT_LAUNCH
+        VMX_CHECK_LAUNCH("window_attention (mixed heads)");
+        return VMX_OK;
+    }
     if (!f32 && seq_starts && num_seqs >= 1 && dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 128 && ldq % 4 == 0 && ((uintptr_t)q & 15) == 0 &&
         ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0) {
         const int qpk = heads / kv_heads, hq = qpk < 4 ? qpk : 4, rt = 16 * (4 / hq);
