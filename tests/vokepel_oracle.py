@@ -55,6 +55,33 @@ def gru_candidate(u):
 
 
 # ------------------------------------------------------------------------------------------------ mixers
+def windowed_attention(q, k, v, scale, size=None, cap=None, r1=None, r2=None, talk=None, sink=None):
+    """q [T, H, D], k [T, G, D], v [T, G, V] of one sequence from its first token.  For every query position i, over the keys j
+    it may see: score = q.k * scale; soft cap; minus r1[h] ln(1 + r2[h] (i - j)); the H scores of a key mixed by talk [H, H];
+    softmax over the keys, the denominator also holding exp(sink[h]); weighted sum of the values.  Returns [T, H, V]."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F)
+    for i in range(T):
+        js = [j for j in range(i + 1) if in_window(i, j, size)]
+        dist = torch.tensor([float(i - j) for j in js], dtype=F)
+        s = torch.zeros(H, len(js), dtype=F)
+        for hh in range(H):
+            g = hh // (H // G)
+            s[hh] = soft_cap((k[js, g] @ q[i, hh]) * scale, cap)
+            if r1 is not None:
+                s[hh] = s[hh] - r1[hh] * torch.log1p(r2[hh] * dist)
+        if talk is not None:
+            s = talk @ s
+        for hh in range(H):
+            g = hh // (H // G)
+            top = s[hh].max() if sink is None else torch.maximum(s[hh].max(), sink[hh])
+            e = torch.exp(s[hh] - top)
+            den = e.sum() + (0.0 if sink is None else torch.exp(sink[hh] - top))
+            out[i, hh] = (e / den) @ v[js, g]
+    return out
+
+
 def biased_talking_attention(h, w, pre, m, eps):
     """Mixer `attention`: values are the un-normed keys, norms over the whole q / k rows, capped scores minus a logarithmic
     distance penalty per head, scores mixed across the heads before the softmax, element-wise output gate."""
@@ -65,25 +92,9 @@ def biased_talking_attention(h, w, pre, m, eps):
     v = k.reshape(T, G, D)
     q = rms_norm(q, w[pre + "q.norm"], eps).reshape(T, H, D)
     k = rms_norm(k, w[pre + "k.norm"], eps).reshape(T, G, D)
-    size = (m.get("mask") or {}).get("size")
-    cap = m.get("softcap")
-    r1, r2, talk = w[pre + "r1"], w[pre + "r2"], w[pre + "talk"]
-    out = torch.zeros(T, H, D, dtype=F)
-    for i in range(T):
-        js = [j for j in range(i + 1) if in_window(i, j, size)]
-        s = torch.zeros(H, len(js), dtype=F)
-        for hh in range(H):
-            g = hh // (H // G)
-            for n, j in enumerate(js):
-                x = soft_cap((q[i, hh] @ k[j, g]) * m["scale"], cap)
-                s[hh, n] = x - r1[hh] * math.log1p(float(r2[hh]) * (i - j))
-        p = torch.softmax(talk @ s, dim=-1)
-        for hh in range(H):
-            g = hh // (H // G)
-            for n, j in enumerate(js):
-                out[i, hh] += p[hh, n] * v[j, g]
-    gate = torch.sigmoid(h @ w[pre + "g"].T)
-    return (out.reshape(T, H * D) * gate) @ w[pre + "o"].T
+    out = windowed_attention(q, k, v, m["scale"], (m.get("mask") or {}).get("size"), m.get("softcap"), w[pre + "r1"], w[pre + "r2"],
+                             w[pre + "talk"])
+    return (out.reshape(T, H * D) * torch.sigmoid(h @ w[pre + "g"].T)) @ w[pre + "o"].T
 
 
 def rotary_sink_attention(h, w, pre, m):
@@ -97,31 +108,25 @@ def rotary_sink_attention(h, w, pre, m):
     if rot:
         q = torch.stack([rotate_pairs(q[t], t, rot["dims"], rot["base"]) for t in range(T)])
         k = torch.stack([rotate_pairs(k[t], t, rot["dims"], rot["base"]) for t in range(T)])
-    size = (m.get("mask") or {}).get("size")
-    out = torch.zeros(T, H, V, dtype=F)
-    for i in range(T):
-        js = [j for j in range(i + 1) if in_window(i, j, size)]
-        for hh in range(H):
-            g = hh // (H // G)
-            s = torch.stack([(q[i, hh] @ k[j, g]) * m["scale"] for j in js])
-            top = max(float(s.max()), float(w[pre + "sink"][hh]))
-            e = torch.exp(s - top)
-            den = e.sum() + math.exp(float(w[pre + "sink"][hh]) - top)
-            for n, j in enumerate(js):
-                out[i, hh] += e[n] / den * v[j, g]
+    out = windowed_attention(q, k, v, m["scale"], (m.get("mask") or {}).get("size"), sink=w[pre + "sink"])
     return out.reshape(T, H * V) @ w[pre + "o"].T
 
 
-def min_gru(h, w, pre):
-    """Right half of mixer `parallel`: S_t = (1 - z_t) S_(t-1) + z_t c_t, gates from the current token only, S_(-1) = 0."""
-    z = torch.sigmoid(h @ w[pre + "z"].T + w[pre + "z.b"])
-    c = gru_candidate(h @ w[pre + "x"].T + w[pre + "x.b"])
-    S = torch.zeros(z.shape[1], dtype=F)
+def min_gru_states(zl, u):
+    """zl, u [T, R]: S_t = (1 - z_t) S_(t-1) + z_t c_t from S = 0, with z = sigmoid(zl) and c the candidate of u.  [T, R]."""
+    z, c = torch.sigmoid(zl), gru_candidate(u)
+    S = torch.zeros(zl.shape[1], dtype=F)
     rows = []
-    for t in range(h.shape[0]):
+    for t in range(zl.shape[0]):
         S = (1.0 - z[t]) * S + z[t] * c[t]
         rows.append(S)
-    return (torch.stack(rows) * silu(h @ w[pre + "g"].T)) @ w[pre + "o"].T
+    return torch.stack(rows)
+
+
+def min_gru(h, w, pre):
+    """Right half of mixer `parallel`: gates from the current token only, SiLU-gated read-out."""
+    S = min_gru_states(h @ w[pre + "z"].T + w[pre + "z.b"], h @ w[pre + "x"].T + w[pre + "x.b"])
+    return (S * silu(h @ w[pre + "g"].T)) @ w[pre + "o"].T
 
 
 def mixer(kind, h, w, pre, m, eps):
