@@ -231,9 +231,10 @@ def test_qk_prepare(gpu, qw, kw_, hd, rot, norms, dtype):
     cdt = torch.float32 if dtype == 0 else torch.bfloat16
     kc, vc = torch.zeros(12, kw_, dtype=cdt, device="cuda"), torch.zeros(12, vw, dtype=cdt, device="cuda")
     inv = torch.tensor([base ** (-2.0 * i / rot) for i in range(rot // 2)], dtype=torch.float32, device="cuda") if rot else None
+    qnd, knd, posd, slotsd = qn.cuda(), kn.cuda(), pos.cuda(), slots.cuda()
     check(lib.vmx_qk_prepare_cache_write(qo.data_ptr(), fused.data_ptr(), ld, qw, fused.data_ptr() + 4 * qw, ld, kw_, fused.data_ptr() + 4 * (qw + kw_), ld,
-                                         vw, qn.cuda().data_ptr() if norms else None, kn.cuda().data_ptr() if norms else None, eps,
-                                         None if inv is None else inv.data_ptr(), rot, hd, pos.cuda().data_ptr(), slots.cuda().data_ptr(),
+                                         vw, qnd.data_ptr() if norms else None, knd.data_ptr() if norms else None, eps,
+                                         None if inv is None else inv.data_ptr(), rot, hd, posd.data_ptr(), slotsd.data_ptr(),
                                          kc.data_ptr(), vc.data_ptr(), dtype, T, None))
     torch.cuda.synchronize()
     qf, kf = q.float().double(), k.float().double()
