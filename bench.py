@@ -864,6 +864,79 @@ def gupuvik_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16))
             "prompt": prompt, "sizes": out}
 
 
+VOKEPEL_SIZES = {
+    # name: (width, heads, kv_heads, dim, window, recurrent width, dense ff, vocab, Gupuvik delta-rule rank)
+    "1k": (1024, 8, 2, 128, 1024, 1024, 4096, 32000, 64),
+    "2k": (2048, 16, 4, 128, 4096, 2048, 8192, 32000, 128),
+}
+
+
+def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16)):
+    """Vokepel (pre-norm layers: rotary sink attention beside a minimal gated recurrent unit / attention with whole-row norms, a
+    distance penalty and mixed heads; squared-ReLU feed-forward; tied, soft-capped logits; bf16 weights) at layer sizes of real
+    models, beside the closest existing model at equal size: Gupuvik, the other packed-step executor with window attention and a
+    recurrent mixer over state slots.  Vokepel: two layers (parallel + dense, attention + dense) looped twice = four layer runs;
+    Gupuvik: four layers (delta rule + dense, attention + dense, twice) with the same width, heads, window, feed-forward width and
+    vocabulary.  Prompt pass: tokens/s of one `prompt`-token sequence; decode: aggregate tok/s of B sequences at context `prompt`,
+    one hipGraph per step."""
+    from vllm_rust_amd.gupuvik import GupuvikForCausalLM, GupuvikLayerSpec, GupuvikSpec
+    from vllm_rust_amd.gupuvik import synthetic_weights as gupuvik_weights
+    from vllm_rust_amd.vokepel import VokepelForCausalLM, VokepelLayerSpec, VokepelSpec, synthetic_weights
+    out = {}
+    dev = torch.device("cuda", torch.cuda.current_device())
+    side = torch.cuda.Stream(device=dev)
+    BM = max(batches)
+    per_seq = (prompt + warmup + steps + 8 + 15) // 16 + 1
+    for name in sizes:
+        W, H, G, dim, win, R, ff, V, rank = VOKEPEL_SIZES[name]
+        sc = 1.0 / math.sqrt(dim)
+        layers = [VokepelLayerSpec(mixer="parallel", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, scale=sc, rot_dims=dim, rot_base=1e6,
+                                   gru_width=R, left_scale=0.6, right_scale=0.5, mlp="dense", ff=ff),
+                  VokepelLayerSpec(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, scale=sc, softcap=50.0, mlp="dense", ff=ff)]
+        spec = VokepelSpec(vocab=V, width=W, layers=layers, residual_mult=0.5, logit_scale=0.5, logit_softcap=15.0, loop=(0, 2, 2))
+        model = VokepelForCausalLM(spec, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+        model.load_state(synthetic_weights(spec, 3, device=dev))
+        t = _packed_times(model, V, prompt, batches, warmup, steps, side, dev, True)
+        model.close()
+        del model
+        hd = H * dim
+        lin_par = W * (hd + 2 * G * dim + 3 * R) + hd * W + R * W + 2 * W * ff
+        lin_att = W * (2 * hd + G * dim) + hd * W + 2 * W * ff
+        lin = 2 * (lin_par + lin_att + 2 * W * W)                 # two passes, each entered through the [x | x0] matrix
+        att_fl = 4 * 2 * H * 2 * dim * min(win, prompt / 2) / 2   # four attention runs, score and value products (MACs)
+        res = {"prefill": {"tokens": prompt, "ms": round(t["prefill"] * 1e3, 3), "tok_s": round(prompt / t["prefill"], 1),
+                           "TFLOP_s": round(2.0 * prompt * (lin + att_fl + V * W / prompt) / t["prefill"] / 1e12, 2)}}
+        wfixed = 2 * ((lin_par + lin_att + 2 * W * W) + V * W)    # bytes of the weights a step reads (looped layers once: the second pass hits cache)
+        for B in batches:
+            by = wfixed + 2 * 4 * B * min(win, prompt + 1) * 2 * G * dim + 2 * 4 * B * R
+            res[f"decode_b{B}"] = {"tok_s": round(B / t[B], 1), "ms_per_step": round(t[B] * 1e3, 4), "GBps_algorithmic": round(by / t[B] / 1e9, 1)}
+        att = dict(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, keep_first=0, scale=sc, softcap=50.0, mlp="dense", ff=ff)
+        dlt = dict(mixer="channel_delta", heads=H, kv_heads=H, dim=dim, vdim=dim, conv=4, decay_rank=rank, gate_rank=rank, mlp="dense", ff=ff)
+        gs = GupuvikSpec(vocab=V, width=W, layers=[GupuvikLayerSpec(**dlt), GupuvikLayerSpec(**att), GupuvikLayerSpec(**dlt), GupuvikLayerSpec(**att)],
+                         embed_scale=1.0)
+        gm = GupuvikForCausalLM(gs, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+        gm.load_state(gupuvik_weights(gs, 3, device=dev))
+        tg = _packed_times(gm, V, prompt, batches, warmup, steps, side, dev, True)
+        gm.close()
+        del gm
+        g_att = W * (hd + 2 * G * dim + H) + hd * W
+        g_dlt = W * (3 * hd + H + 2 * rank) + rank * 2 * hd + hd * W
+        glin = 2 * (g_att + g_dlt + 2 * 2 * W * W + 2 * 2 * W * ff)
+        gres = {"prefill": {"tokens": prompt, "ms": round(tg["prefill"] * 1e3, 3), "tok_s": round(prompt / tg["prefill"], 1),
+                            "TFLOP_s": round(2.0 * prompt * (glin + 2 * H * 2 * dim * min(win, prompt / 2) + 2 * H * 3 * dim * dim + V * W / prompt)
+                                             / tg["prefill"] / 1e12, 2)}}
+        gfixed = 2 * (glin + 2 * V * W)
+        for B in batches:
+            by = gfixed + 2 * 2 * B * min(win, prompt + 1) * 2 * G * dim + 2 * 2 * B * H * dim * dim * 4
+            gres[f"decode_b{B}"] = {"tok_s": round(B / tg[B], 1), "ms_per_step": round(tg[B] * 1e3, 4), "GBps_algorithmic": round(by / tg[B] / 1e9, 1)}
+        out[name] = {"vokepel": res, "gupuvik": gres,
+                     "config": {"width": W, "layers": ["parallel+dense", "attention+dense"], "loop": [0, 2, 2], "heads": H, "kv_heads": G, "dim": dim,
+                                "window": win, "gru_width": R, "ff": ff, "vocab": V,
+                                "gupuvik": {"layers": ["channel_delta+dense", "attention+dense"] * 2, "rank": rank, "conv": 4}}}
+    return {"metric": "Vokepel prompt and decode throughput beside Gupuvik at equal size", "unit": "tok/s", "dtype": "bf16", "data": "synthetic",
+            "prompt": prompt, "sizes": out}
+
+
 def plan_job(gpus, world, replicas_flag, weights, local_ranks):
     """What a launch of this script measures -- pure argument logic, no device.  N = 1: the single-GPU job.  N > 1 (one process
     per GPU under torch.distributed.run): ONE model tensor-parallel over the N ranks (BASELINE.json's metric is the TP curve at
@@ -1020,13 +1093,14 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary measurements (other models at N = 1, replicas at N > 1)")
     ap.add_argument("--no-moe", action="store_true", help="skip the Mixtral-8x7B-shaped fused-MoE secondary measurement")
-    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar", "gupuvik"], default="all",
+    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel"], default="all",
                     help="profiling aid: run ONE workload alone (qwen3 = the primary without secondaries; the others print only "
                          "their own block), so that a kernel trace of the run holds that workload's launches only; gesutar = the Gesutar "
                          "executor (latent attention + grouped-router MoE, bf16) at two layer sizes beside the bf16 dense Qwen3 executor at "
                          "equal size: prompt tok/s and decode tok/s at 1 and 16 sequences (not part of the default run); gupuvik = the Gupuvik "
                          "executor (window attention / gated delta rule, gated residuals, bf16) at two layer sizes beside Gesutar at equal size, "
-                         "the same measurements")
+                         "the same measurements; vokepel = the Vokepel executor (looped pre-norm layers, rotary sink attention beside a minimal "
+                         "gated recurrent unit, mixed-head attention, bf16) at two layer sizes beside Gupuvik at equal size, the same measurements")
     ap.add_argument("--tp", action="store_true", help="accepted for compatibility: with --gpus N > 1 the tensor-parallel job is the default")
     ap.add_argument("--replicas", action="store_true",
                     help="with --gpus N > 1: N independent replicas as the primary (weak scaling, no collective) instead of ONE model "
@@ -1041,8 +1115,10 @@ def main():
     plan = plan_job(args.gpus, world, args.replicas, args.weights, d.local)
 
     K_steps, W_steps = args.steps, args.warmup
-    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar", "gupuvik"):   # one secondary alone (single GPU)
-        if args.workload == "gupuvik":
+    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel"):   # one secondary alone (single GPU)
+        if args.workload == "vokepel":
+            blk = vokepel_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
+        elif args.workload == "gupuvik":
             blk = gupuvik_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
         elif args.workload == "gesutar":
             blk = gesutar_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)

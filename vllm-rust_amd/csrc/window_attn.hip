@@ -546,6 +546,305 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
         }
 }
 
+// Matrix-core form with mixed heads (bf16 cache).  A workgroup of 8 waves owns 16 consecutive rows of ONE sequence and ALL heads:
+// wave w the heads w, w + 8, ... (HPW of them).  The visible keys are walked in tiles of 32; the key rows of every key/value head
+// are staged row-major in LDS and the value rows transposed (keys permuted as in the form above), one tile ahead through registers.
+// Per tile: (A) every wave computes S^T = K Q^T of its heads, shapes the scores (scale, soft cap, distance penalty) and leaves them
+// in LDS as raw[head][query][key]; (B) it reads the scores of ALL heads at its lanes' (query, key) places, mixes them with its
+// heads' rows of the mixing matrix, and goes on per head as above: mask, running softmax in the four lanes of a query,
+// O^T += V^T P^T with P as a bf16 pair.  Launches of few rows deal a run's key tiles to several workgroups (merge kernel below).
+constexpr int TM_KT = 32, TM_NW = 8, TM_NT = 64 * TM_NW, TM_MAXCH = 4;
+__host__ __device__ constexpr int tm_ldk(int ds) { return 32 * ds + 8; }
+static size_t talk_mfma_lds_bytes(int heads, int kv_heads, int ds, int vs) {
+    return (size_t)kv_heads * TM_KT * tm_ldk(ds) * 2 + (size_t)kv_heads * 16 * vs * (TM_KT + 8) * 2 + (size_t)heads * 16 * (TM_KT + 4) * 4 +
+           (size_t)heads * heads * 4;
+}
+
+template <int DS, int VS, int HPW>
+__global__ __launch_bounds__(TM_NT) void talk_attn_mfma_kernel(const WinAttn p) {
+    constexpr int KT = TM_KT, NW = TM_NW, NT = TM_NT, LDK = tm_ldk(DS), LDV = KT + 8, LDR = KT + 4, MAXCH = TM_MAXCH;
+    extern __shared__ __align__(16) unsigned char talk_mfma_lds[];
+    const int H = p.heads, G = p.kv_heads, D = p.dim, V = p.vdim, qpk = H / G;
+    uint16_t *Ks = (uint16_t *)talk_mfma_lds;             // [G][KT][LDK]
+    uint16_t *Vt = Ks + G * KT * LDK;                     // [G][16 VS][LDV]
+    float *raw = (float *)(Vt + G * 16 * VS * LDV);       // [H][16][LDR]
+    float *tk = raw + H * 16 * LDR;                       // [H][H]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fl = lane & 15, fg = lane >> 4;
+    const int share = blockIdx.x % p.parts;
+    int tile = blockIdx.x / p.parts, r0 = 0, nrows = 0;
+    for (int s = 0; s < p.num_seqs; s++) {
+        const int a = p.seq_starts[s], len = p.seq_starts[s + 1] - a, n = (len + 15) / 16;
+        if (tile < n) {
+            r0 = a + tile * 16;
+            nrows = min(16, len - tile * 16);
+            break;
+        }
+        tile -= n;
+    }
+    if (nrows <= 0) return;   // the same for the whole workgroup
+    const int64_t kw = (int64_t)G * D, vw = (int64_t)G * V;
+    const int i0 = p.positions[r0], i1 = i0 + nrows - 1;
+    const int lo = p.window > 0 ? max(0, i0 - p.window + 1) : 0;
+    const int na = min(p.keep_first, lo), nk = na + (i1 - lo + 1);
+    const int32_t *bt = p.block_tables + (int64_t)p.seq_ids[r0] * p.max_blocks;
+    const uint16_t *kc = (const uint16_t *)p.kc, *vc = (const uint16_t *)p.vc;
+    const int qi = i0 + fl;
+    const bool qlive = fl < nrows;
+    uint4 qf[HPW][DS];
+    float smul[HPW], dr1[HPW], dr2[HPW];
+#pragma unroll
+    for (int a = 0; a < HPW; a++) {
+        const int h = wave + NW * a;
+        const bool on = h < H;
+        smul[a] = p.scale * (p.temp && on ? vmx_bf16_to_f32(p.temp[h]) : 1.0f);
+        dr1[a] = p.r1 && on ? vmx_bf16_to_f32(p.r1[h]) : 0.f;
+        dr2[a] = p.r1 && on ? vmx_bf16_to_f32(p.r2[h]) : 0.f;
+#pragma unroll
+        for (int s = 0; s < DS; s++) {
+            const int k = 32 * s + 8 * fg;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (on && qlive && k < D) {
+                const float *src = p.q + (int64_t)(r0 + fl) * p.ldq + (int64_t)h * D + k;
+                float f[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) f[e] = src[e];
+                v = vmx_pack16x8<false>(f);
+            }
+            qf[a][s] = v;
+        }
+    }
+    for (int i = tid; i < H * H; i += NT) tk[i] = vmx_bf16_to_f32(p.talk[i]);
+    const float inv_cap = p.softcap > 0.f ? 1.0f / p.softcap : 0.f;
+    const int ntile = (nk + KT - 1) / KT, per = (ntile + p.parts - 1) / p.parts;
+    const int kb0 = share * per * KT, kb1 = min(nk, (share + 1) * per * KT);
+    const int nKch = KT * G * 4 * DS, nVch = KT * G * 2 * VS;
+    uint4 kr[MAXCH], vr[MAXCH];
+    int krow[MAXCH], vrow[MAXCH];
+    auto cache_row = [&](int idx) -> int {
+        if (idx >= nk) return 0;
+        const int j = idx < na ? idx : lo + (idx - na);
+        if (p.bs_shift >= 0) return (bt[j >> p.bs_shift] << p.bs_shift) + (j & (p.block_size - 1));
+        return bt[j / p.block_size] * p.block_size + j % p.block_size;
+    };
+    auto lookup = [&](int kb) {
+#pragma unroll
+        for (int c = 0; c < MAXCH; c++) {
+            const int ch = tid + NT * c;
+            krow[c] = cache_row(kb + (ch / (4 * DS)) % KT);
+            vrow[c] = cache_row(kb + ch % KT);
+        }
+    };
+    auto fetch = [&](int kb) {
+#pragma unroll
+        for (int c = 0; c < MAXCH; c++) {
+            const int ch = tid + NT * c;
+            {
+                const int part = ch % (4 * DS), kk = (ch / (4 * DS)) % KT, g = ch / (4 * DS * KT);
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (ch < nKch && kb + kk < kb1 && 8 * part < D) v = *reinterpret_cast<const uint4 *>(kc + (int64_t)krow[c] * kw + (int64_t)g * D + 8 * part);
+                kr[c] = v;
+            }
+            {
+                const int kk = ch % KT, part = (ch / KT) % (2 * VS), g = ch / (KT * 2 * VS);
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (ch < nVch && kb + kk < kb1 && 8 * part < V) v = *reinterpret_cast<const uint4 *>(vc + (int64_t)vrow[c] * vw + (int64_t)g * V + 8 * part);
+                vr[c] = v;
+            }
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int c = 0; c < MAXCH; c++) {
+            const int ch = tid + NT * c;
+            if (ch < nKch) {
+                const int part = ch % (4 * DS), kk = (ch / (4 * DS)) % KT, g = ch / (4 * DS * KT);
+                *reinterpret_cast<uint4 *>(Ks + (g * KT + kk) * LDK + 8 * part) = kr[c];
+            }
+            if (ch < nVch) {
+                const int kk = ch % KT, part = (ch / KT) % (2 * VS), g = ch / (KT * 2 * VS);
+                const int col = 8 * ((kk & 15) >> 2) + (kk & 3) + 4 * ((kk >> 4) & 1);   // the k slot in which the score registers meet key kk
+                const uint32_t w[4] = {vr[c].x, vr[c].y, vr[c].z, vr[c].w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) Vt[(g * 16 * VS + 8 * part + e) * LDV + col] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    };
+    float m[HPW], den[HPW];
+    vmx_f32x4 o[HPW][VS];
+#pragma unroll
+    for (int a = 0; a < HPW; a++) {
+        m[a] = -FLT_MAX, den[a] = 0.f;
+#pragma unroll
+        for (int v = 0; v < VS; v++) o[a][v] = vmx_f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    lookup(kb0);
+    fetch(kb0);
+    lookup(kb0 + KT);
+    stash();
+    __syncthreads();
+    for (int kb = kb0; kb < kb1; kb += KT) {
+        if (kb + KT < kb1) {
+            fetch(kb + KT);
+            lookup(kb + 2 * KT);
+        }
+        // (A) shaped scores of this wave's heads into LDS
+#pragma unroll
+        for (int a = 0; a < HPW; a++) {
+            const int h = wave + NW * a;
+            if (h < H) {
+                const int g = h / qpk;
+#pragma unroll
+                for (int kt = 0; kt < KT / 16; kt++) {
+                    vmx_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < DS; s++) {
+                        const uint4 ka = *reinterpret_cast<const uint4 *>(Ks + (g * KT + 16 * kt + fl) * LDK + 32 * s + 8 * fg);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, ka), __builtin_bit_cast(vmx_bf16x8, qf[a][s]), acc, 0, 0, 0);
+                    }
+                    float4 x4;
+                    float *xs = &x4.x;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int idx = kb + 16 * kt + 4 * fg + r;
+                        const int j = idx < na ? idx : lo + (idx - na);
+                        float x = acc[r] * smul[a];
+                        if (p.softcap > 0.f) x = p.softcap * tanh_fast(x * inv_cap);
+                        if (p.r1) x -= dr1[a] * __logf(1.0f + dr2[a] * (float)max(qi - j, 0));
+                        xs[r] = x;
+                    }
+                    *reinterpret_cast<float4 *>(raw + (h * 16 + fl) * LDR + 16 * kt + 4 * fg) = x4;
+                }
+            }
+        }
+        __syncthreads();
+        // (B) mixed scores of this wave's heads, softmax, weighted values
+#pragma unroll
+        for (int a = 0; a < HPW; a++) {
+            const int h = wave + NW * a;
+            if (h < H) {
+                const int g = h / qpk;
+                float sc[KT / 16][4];
+                float tmax = -FLT_MAX;
+#pragma unroll
+                for (int kt = 0; kt < KT / 16; kt++) {
+                    float4 mix = make_float4(0.f, 0.f, 0.f, 0.f);
+                    for (int g2 = 0; g2 < H; g2++) {
+                        const float t = tk[h * H + g2];
+                        const float4 r4 = *reinterpret_cast<const float4 *>(raw + (g2 * 16 + fl) * LDR + 16 * kt + 4 * fg);
+                        mix.x = fmaf(t, r4.x, mix.x), mix.y = fmaf(t, r4.y, mix.y), mix.z = fmaf(t, r4.z, mix.z), mix.w = fmaf(t, r4.w, mix.w);
+                    }
+                    const float mx[4] = {mix.x, mix.y, mix.z, mix.w};
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int idx = kb + 16 * kt + 4 * fg + r;
+                        const int j = idx < na ? idx : lo + (idx - na);
+                        const bool vis = qlive && idx < kb1 && j <= qi && (p.window == 0 || qi - j < p.window || j < p.keep_first);
+                        sc[kt][r] = vis ? mx[r] : -FLT_MAX;
+                        tmax = fmaxf(tmax, sc[kt][r]);
+                    }
+                }
+                tmax = fmaxf(tmax, vmx_lane_xor<16>(tmax));
+                tmax = fmaxf(tmax, vmx_lane_xor<32>(tmax));
+                const float mn = fmaxf(m[a], tmax);
+                const float f = __expf(m[a] - mn);
+                float psum = 0.f;
+#pragma unroll
+                for (int kt = 0; kt < KT / 16; kt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        sc[kt][r] = sc[kt][r] > -FLT_MAX ? __expf(sc[kt][r] - mn) : 0.f;
+                        psum += sc[kt][r];
+                    }
+                psum += vmx_lane_xor<16>(psum);
+                psum += vmx_lane_xor<32>(psum);
+                den[a] = den[a] * f + psum;
+                m[a] = mn;
+                if (__any(f != 1.0f)) {
+#pragma unroll
+                    for (int v = 0; v < VS; v++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) o[a][v][r] *= f;
+                }
+                float hi[8], lw[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float pv = sc[e >> 2][e & 3];
+                    hi[e] = vmx_bf16_to_f32(vmx_f32_to_bf16(pv));
+                    lw[e] = pv - hi[e];
+                }
+                const uint4 bh = vmx_pack16x8<false>(hi), bl = vmx_pack16x8<false>(lw);
+#pragma unroll
+                for (int v = 0; v < VS; v++) {
+                    const uint4 va = *reinterpret_cast<const uint4 *>(Vt + (g * 16 * VS + 16 * v + fl) * LDV + 8 * fg);
+                    o[a][v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, va), __builtin_bit_cast(vmx_bf16x8, bh), o[a][v], 0, 0, 0);
+                    o[a][v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, va), __builtin_bit_cast(vmx_bf16x8, bl), o[a][v], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+        if (kb + KT < kb1) {
+            stash();
+            __syncthreads();
+        }
+    }
+    if (!qlive) return;
+#pragma unroll
+    for (int a = 0; a < HPW; a++) {
+        const int h = wave + NW * a;
+        if (h >= H) continue;
+        if (p.parts > 1) {
+            float *w = p.ws + (((int64_t)(r0 + fl) * H + h) * p.parts + share) * (V + 2);
+#pragma unroll
+            for (int v = 0; v < VS; v++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int c = 16 * v + 4 * fg + r;
+                    if (c < V) w[c] = o[a][v][r];
+                }
+            if (fg == 0) w[V] = m[a], w[V + 1] = den[a];
+            continue;
+        }
+        if (p.sink) {
+            float f;
+            add_sink(vmx_bf16_to_f32(p.sink[h]), m[a], den[a], f);
+#pragma unroll
+            for (int v = 0; v < VS; v++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[a][v][r] *= f;
+        }
+        float gsc = 1.0f / den[a];
+        if (p.gate && !p.gate_elem) gsc *= sigmoid_f32(p.gate[(int64_t)(r0 + fl) * p.ldgate + h]);
+#pragma unroll
+        for (int v = 0; v < VS; v++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int c = 16 * v + 4 * fg + r;
+                if (c < V) {
+                    const int64_t at = ((int64_t)(r0 + fl) * H + h) * V + c;
+                    float x = o[a][v][r] * gsc;
+                    if (p.gate && p.gate_elem) x *= sigmoid_f32(p.gate[(int64_t)(r0 + fl) * p.ldgate + (int64_t)h * V + c]);
+                    if (p.out_f32) ((float *)p.out)[at] = x;
+                    else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(x);
+                }
+            }
+    }
+}
+
+template <int DS, int VS, int HPW> int talk_mfma_launch(const WinAttn &p, dim3 grid, size_t lds, hipStream_t st) {
+    static bool sized = false;
+    if (!sized) {
+        VMX_CHECK_HIP(hipFuncSetAttribute((const void *)talk_attn_mfma_kernel<DS, VS, HPW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        sized = true;
+    }
+    hipLaunchKernelGGL((talk_attn_mfma_kernel<DS, VS, HPW>), grid, dim3(TM_NT), lds, st, p);
+    return VMX_OK;
+}
+template <int DS, int VS> int talk_mfma_launch_h(int hpw, const WinAttn &p, dim3 grid, size_t lds, hipStream_t st) {
+    if (hpw == 1) return talk_mfma_launch<DS, VS, 1>(p, grid, lds, st);
+    if (hpw == 2) return talk_mfma_launch<DS, VS, 2>(p, grid, lds, st);
+    return talk_mfma_launch<DS, VS, 4>(p, grid, lds, st);
+}
+
 // out[t, h] = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) den_p * sigmoid(gate): the shares of a row's keys put together.  One wave
 // per row: lane p takes share p's maximum and denominator (at most 16 shares), the weights are then handed round by lane reads.
 __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) {
@@ -653,6 +952,35 @@ extern "C" int vmx_window_attention_ex(void *out, int out_dtype, const float *q,
               ex.sink_bf16, ex.dist_r1_bf16, ex.dist_r2_bf16, ex.talk_bf16, ex.gate_per_element ? 1 : 0};
     hipStream_t st = vmx_stream(stream);
     const bool f32 = cache_dtype == VMX_F32;
+    if (p.talk && !f32 && seq_starts && num_seqs >= 1 && dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 128 && ldq % 4 == 0 &&
+        ((uintptr_t)q & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0 && heads <= 4 * TM_NW) {
+        // all heads of 16 rows in one workgroup, on the matrix cores, when the tiles of all key/value heads fit
+        const int ds = dim <= 64 ? 2 : (dim <= 128 ? 4 : 8), vs = vdim <= 32 ? 2 : (vdim <= 64 ? 4 : 8);
+        const int hpw = (heads + TM_NW - 1) / TM_NW, hp = hpw <= 2 ? hpw : 4;
+        const size_t lds = talk_mfma_lds_bytes(heads, kv_heads, ds, vs);
+        const bool fits = (size_t)TM_KT * kv_heads * 4 * ds <= (size_t)TM_MAXCH * TM_NT && (size_t)TM_KT * kv_heads * 2 * vs <= (size_t)TM_MAXCH * TM_NT &&
+                          lds <= 160 * 1024 && hp * (ds + vs) <= 40;   // staging registers, LDS, and the registers of a wave's heads
+        if (fits) {
+            const int runs = tokens / 16 + num_seqs;
+            if (workspace && runs < 128) {
+                int parts = 256 / runs < 16 ? 256 / runs : 16;
+                if (window > 0) parts = std::min(parts, (window + keep_first + 16 + TM_KT - 1) / TM_KT);
+                parts = std::min<size_t>(parts, workspace_bytes / ((size_t)tokens * heads * (vdim + 2) * 4));
+                if (parts > 1) p.parts = parts;
+            }
+            const dim3 grid(runs * p.parts);
+            int rc;
+#define TM_V(A)                                                              \
+    (vs == 2 ? talk_mfma_launch_h<A, 2>(hp, p, grid, lds, st) : vs == 4 ? talk_mfma_launch_h<A, 4>(hp, p, grid, lds, st) \
+                                                                         : talk_mfma_launch_h<A, 8>(hp, p, grid, lds, st))
+            rc = ds == 2 ? TM_V(2) : (ds == 4 ? TM_V(4) : TM_V(8));
+#undef TM_V
+            if (rc) return rc;
+            if (p.parts > 1) hipLaunchKernelGGL(window_attn_merge_kernel, dim3(tokens * heads), dim3(64), 0, st, p);
+            VMX_CHECK_LAUNCH("window_attention (mixed heads, matrix cores)");
+            return VMX_OK;
+        }
+    }
     if (p.talk) {   // all heads of a token in one workgroup
         const int nw = heads < 8 ? heads : 8, hpw = (heads + nw - 1) / nw;
         const int vpl = vdim <= 64 ? 1 : (vdim <= 128 ? 2 : 4);
