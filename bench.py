@@ -871,7 +871,7 @@ VOKEPEL_SIZES = {
 }
 
 
-def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16)):
+def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16), comparator=True):
     """Vokepel (pre-norm layers: rotary sink attention beside a minimal gated recurrent unit / attention with whole-row norms, a
     distance penalty and mixed heads; squared-ReLU feed-forward; tied, soft-capped logits; bf16 weights) at layer sizes of real
     models, beside the closest existing model at equal size: Gupuvik, the other packed-step executor with window attention and a
@@ -910,6 +910,9 @@ def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16))
         for B in batches:
             by = wfixed + 2 * 4 * B * min(win, prompt + 1) * 2 * G * dim + 2 * 4 * B * R
             res[f"decode_b{B}"] = {"tok_s": round(B / t[B], 1), "ms_per_step": round(t[B] * 1e3, 4), "GBps_algorithmic": round(by / t[B] / 1e9, 1)}
+        if not comparator:
+            out[name] = {"vokepel": res}
+            continue
         att = dict(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, keep_first=0, scale=sc, softcap=50.0, mlp="dense", ff=ff)
         dlt = dict(mixer="channel_delta", heads=H, kv_heads=H, dim=dim, vdim=dim, conv=4, decay_rank=rank, gate_rank=rank, mlp="dense", ff=ff)
         gs = GupuvikSpec(vocab=V, width=W, layers=[GupuvikLayerSpec(**dlt), GupuvikLayerSpec(**att), GupuvikLayerSpec(**dlt), GupuvikLayerSpec(**att)],
@@ -1093,6 +1096,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary measurements (other models at N = 1, replicas at N > 1)")
     ap.add_argument("--no-moe", action="store_true", help="skip the Mixtral-8x7B-shaped fused-MoE secondary measurement")
+    ap.add_argument("--no-comparator", action="store_true", help="--workload vokepel: time the Vokepel executor alone (kernel traces of one model)")
+    ap.add_argument("--sizes", default="1k,2k", help="--workload vokepel: which of its sizes to run")
     ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel"], default="all",
                     help="profiling aid: run ONE workload alone (qwen3 = the primary without secondaries; the others print only "
                          "their own block), so that a kernel trace of the run holds that workload's launches only; gesutar = the Gesutar "
@@ -1117,7 +1122,8 @@ def main():
     K_steps, W_steps = args.steps, args.warmup
     if args.workload in ("gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel"):   # one secondary alone (single GPU)
         if args.workload == "vokepel":
-            blk = vokepel_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
+            blk = vokepel_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup,
+                                   sizes=tuple(args.sizes.split(",")), comparator=not args.no_comparator)
         elif args.workload == "gupuvik":
             blk = gupuvik_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
         elif args.workload == "gesutar":

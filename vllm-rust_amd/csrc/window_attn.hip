@@ -557,7 +557,7 @@ constexpr int TM_KT = 32, TM_NW = 8, TM_NT = 64 * TM_NW, TM_MAXCH = 4;
 __host__ __device__ constexpr int tm_ldk(int ds) { return 32 * ds + 8; }
 static size_t talk_mfma_lds_bytes(int heads, int kv_heads, int ds, int vs) {
     return (size_t)kv_heads * TM_KT * tm_ldk(ds) * 2 + (size_t)kv_heads * 16 * vs * (TM_KT + 8) * 2 + (size_t)heads * 16 * (TM_KT + 4) * 4 +
-           (size_t)heads * heads * 4;
+           (size_t)heads * ((heads + 3) & ~3) * 4;
 }
 
 template <int DS, int VS, int HPW>
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(TM_NT) void talk_attn_mfma_kernel(const WinAttn p) 
     uint16_t *Ks = (uint16_t *)talk_mfma_lds;             // [G][KT][LDK]
     uint16_t *Vt = Ks + G * KT * LDK;                     // [G][16 VS][LDV]
     float *raw = (float *)(Vt + G * 16 * VS * LDV);       // [H][16][LDR]
-    float *tk = raw + H * 16 * LDR;                       // [H][H]
+    float *tk = raw + H * 16 * LDR;                       // [H][H rounded up to 4]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fl = lane & 15, fg = lane >> 4;
     const int share = blockIdx.x % p.parts;
     int tile = blockIdx.x / p.parts, r0 = 0, nrows = 0;
@@ -613,7 +613,8 @@ __global__ __launch_bounds__(TM_NT) void talk_attn_mfma_kernel(const WinAttn p) 
             qf[a][s] = v;
         }
     }
-    for (int i = tid; i < H * H; i += NT) tk[i] = vmx_bf16_to_f32(p.talk[i]);
+    const int H4 = (H + 3) & ~3;   // rows of the mixing matrix padded with zeros to whole float4s
+    for (int i = tid; i < H * H4; i += NT) tk[i] = i % H4 < H ? vmx_bf16_to_f32(p.talk[(i / H4) * H + i % H4]) : 0.f;
     const float inv_cap = p.softcap > 0.f ? 1.0f / p.softcap : 0.f;
     const int ntile = (nk + KT - 1) / KT, per = (ntile + p.parts - 1) / p.parts;
     const int kb0 = share * per * KT, kb1 = min(nk, (share + 1) * per * KT);
@@ -727,11 +728,19 @@ __global__ __launch_bounds__(TM_NT) void talk_attn_mfma_kernel(const WinAttn p) 
                 float tmax = -FLT_MAX;
 #pragma unroll
                 for (int kt = 0; kt < KT / 16; kt++) {
+                    // four heads' scores and weights are requested together, so that their LDS trips overlap
                     float4 mix = make_float4(0.f, 0.f, 0.f, 0.f);
-                    for (int g2 = 0; g2 < H; g2++) {
-                        const float t = tk[h * H + g2];
-                        const float4 r4 = *reinterpret_cast<const float4 *>(raw + (g2 * 16 + fl) * LDR + 16 * kt + 4 * fg);
-                        mix.x = fmaf(t, r4.x, mix.x), mix.y = fmaf(t, r4.y, mix.y), mix.z = fmaf(t, r4.z, mix.z), mix.w = fmaf(t, r4.w, mix.w);
+                    for (int g2 = 0; g2 < H; g2 += 4) {
+                        const float4 t4 = *reinterpret_cast<const float4 *>(tk + h * H4 + g2);
+                        float4 r4[4];
+#pragma unroll
+                        for (int u = 0; u < 4; u++)   // past the last head: its row again, under a zero weight
+                            r4[u] = *reinterpret_cast<const float4 *>(raw + (min(g2 + u, H - 1) * 16 + fl) * LDR + 16 * kt + 4 * fg);
+                        const float tw[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+                        for (int u = 0; u < 4; u++)
+                            mix.x = fmaf(tw[u], r4[u].x, mix.x), mix.y = fmaf(tw[u], r4[u].y, mix.y), mix.z = fmaf(tw[u], r4[u].z, mix.z),
+                            mix.w = fmaf(tw[u], r4[u].w, mix.w);
                     }
                     const float mx[4] = {mix.x, mix.y, mix.z, mix.w};
 #pragma unroll
@@ -846,7 +855,7 @@ template <int DS, int VS> int talk_mfma_launch_h(int hpw, const WinAttn &p, dim3
 }
 
 // out[t, h] = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) den_p * sigmoid(gate): the shares of a row's keys put together.  One wave
-// per row: lane p takes share p's maximum and denominator (at most 16 shares), the weights are then handed round by lane reads.
+// per row: lane p takes share p's maximum and denominator (at most 32 shares), the weights are then handed round by lane reads.
 __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) {
     const int row = blockIdx.x, t = row / p.heads, h = row % p.heads, V = p.vdim, lane = threadIdx.x;
     const float *w = p.ws + (int64_t)row * p.parts * (V + 2);
@@ -859,12 +868,14 @@ __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) 
     if (p.gate && !p.gate_elem) g *= sigmoid_f32(p.gate[(int64_t)t * p.ldgate + h]);
     for (int c0 = 0; c0 < V; c0 += 64) {
         const int c = c0 + lane, cc = min(c, V - 1);
-        float x[16];                                       // every share's value first: independent loads, one wait
-#pragma unroll
-        for (int q = 0; q < 16; q++) x[q] = q < p.parts ? w[q * (V + 2) + cc] : 0.f;
         float acc = 0.f;
+        for (int q0 = 0; q0 < p.parts; q0 += 16) {         // sixteen shares' values first: independent loads, one wait
+            float x[16];
 #pragma unroll
-        for (int q = 0; q < 16; q++) acc = fmaf(__shfl(eq, q, 64), x[q], acc);
+            for (int q = 0; q < 16; q++) x[q] = q0 + q < p.parts ? w[(q0 + q) * (V + 2) + cc] : 0.f;
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc = fmaf(__shfl(eq, q0 + q, 64), x[q], acc);
+        }
         if (c < V) {
             const int64_t at = (int64_t)row * V + c;
             float r = acc * g;
@@ -878,8 +889,8 @@ __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) 
 }  // namespace
 
 extern "C" size_t vmx_window_attention_workspace_bytes(int tokens, int heads, int vdim) {
-    // enough for 16 shares of up to 256 rows: launches with more rows fill the chip without splitting their keys
-    return (size_t)(tokens < 256 ? tokens : 256) * heads * 16 * (vdim + 2) * 4;
+    // enough for 32 shares of up to 256 rows: launches with more rows fill the chip without splitting their keys
+    return (size_t)(tokens < 256 ? tokens : 256) * heads * 32 * (vdim + 2) * 4;
 }
 
 extern "C" int vmx_kv_cache_write_f32(const float *k, int64_t ldk, const float *v, int64_t ldv, const int32_t *slots, void *k_cache,
@@ -963,7 +974,7 @@ extern "C" int vmx_window_attention_ex(void *out, int out_dtype, const float *q,
         if (fits) {
             const int runs = tokens / 16 + num_seqs;
             if (workspace && runs < 128) {
-                int parts = 256 / runs < 16 ? 256 / runs : 16;
+                int parts = 256 / runs < 32 ? 256 / runs : 32;   // one workgroup holds all heads: a run has few workgroups to begin with
                 if (window > 0) parts = std::min(parts, (window + keep_first + 16 + TM_KT - 1) / TM_KT);
                 parts = std::min<size_t>(parts, workspace_bytes / ((size_t)tokens * heads * (vdim + 2) * 4));
                 if (parts > 1) p.parts = parts;
