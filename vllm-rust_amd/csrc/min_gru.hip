@@ -4,27 +4,29 @@
 // zeros, so a slot is never cleared when it changes hands.  Everything here is f32.
 //
 // The recurrence is linear in S, S_t = a_t S_(t-1) + b_t, so a run of rows composes to one pair (A, B) = (prod a, the run's result
-// from a zero start) and runs can be walked side by side: a workgroup owns 64 channels of one sequence and 16 strands (waves),
-// strand s the s-th sixteenth of the sequence's rows.  Pass 1: every strand composes its run; pass 2: it starts from the slot's
-// state pushed through the pairs of the strands before it and walks its rows again, now storing y.  A decode step is the case of
-// one row: strand 0 works, the others hold the identity.  A row's result depends on where the strands' borders fall only by f32
-// rounding of the composition.
+// from a zero start) and runs can be walked side by side: a workgroup owns 16 channels of one sequence and 64 strands (a wave
+// holds four of them: 64-byte pieces of four rows per load), strand s the s-th 64th of the sequence's rows.  Pass 1: every strand
+// composes its run; pass 2: it starts from the slot's state pushed through the pairs of the strands before it and walks its rows
+// again, now storing y.  Steps whose runs are at most four rows long (decode) take the one-strand form: a thread per (sequence,
+// channel), 256 channels a workgroup.  A row's result depends on where the strands' borders fall only by f32 rounding of the
+// composition.
 #include "vmx_kernels.h"
 
 namespace {
 
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-constexpr int GRU_STRANDS = 16;
-
-__global__ __launch_bounds__(64 * GRU_STRANDS) void min_gru_kernel(void *__restrict__ y, int y_f32, const float *__restrict__ zl, int64_t ldz,
+// <16 channels, 64 strands> for steps with prompt portions; <256, 1> when every sequence brings at most one row per strand anyway
+// (decode steps: tokens - sequences + 1 bounds the longest run)
+template <int GRU_CH, int GRU_STRANDS>
+__global__ __launch_bounds__(GRU_CH * GRU_STRANDS) void min_gru_kernel(void *__restrict__ y, int y_f32, const float *__restrict__ zl, int64_t ldz,
                                                                    const float *__restrict__ u, int64_t ldu, const float *__restrict__ g,
                                                                    int64_t ldg, float *__restrict__ state, const int32_t *__restrict__ positions,
                                                                    const int32_t *__restrict__ seq_starts, const int32_t *__restrict__ state_slots,
                                                                    int width) {
-    __shared__ float As[GRU_STRANDS][64], Bs[GRU_STRANDS][64];
-    const int lane = threadIdx.x & 63, strand = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + lane, s = blockIdx.y;
+    __shared__ float As[GRU_STRANDS][GRU_CH], Bs[GRU_STRANDS][GRU_CH];
+    const int lane = threadIdx.x % GRU_CH, strand = threadIdx.x / GRU_CH;
+    const int c = blockIdx.x * GRU_CH + lane, s = blockIdx.y;
     const int r0 = seq_starts[s], len = seq_starts[s + 1] - r0;
     if (len <= 0) return;   // the same for the whole workgroup
     const bool live = c < width;
@@ -74,8 +76,13 @@ extern "C" int vmx_min_gru(void *y, int y_dtype, const float *zl, int64_t ldz, c
     VMX_REQUIRE(width >= 1 && ldz >= width && ldu >= width && (!g || ldg >= width), "min_gru: bad width or row strides");
     VMX_REQUIRE(num_seqs >= 0 && num_seqs <= 65535, "min_gru: %d sequences in one step", num_seqs);
     if (num_seqs == 0 || tokens <= 0) return VMX_OK;
-    hipLaunchKernelGGL(min_gru_kernel, dim3((width + 63) / 64, num_seqs), dim3(64 * GRU_STRANDS), 0, vmx_stream(stream), y, y_dtype == VMX_F32, zl,
-                       ldz, u, ldu, g, ldg, state, positions, seq_starts, state_slots, width);
+    hipStream_t st = vmx_stream(stream);
+    if (tokens - num_seqs + 1 <= 4)   // no run longer than four rows
+        hipLaunchKernelGGL((min_gru_kernel<256, 1>), dim3((width + 255) / 256, num_seqs), dim3(256), 0, st, y, y_dtype == VMX_F32, zl, ldz, u, ldu, g, ldg,
+                           state, positions, seq_starts, state_slots, width);
+    else
+        hipLaunchKernelGGL((min_gru_kernel<16, 64>), dim3((width + 15) / 16, num_seqs), dim3(1024), 0, st, y, y_dtype == VMX_F32, zl, ldz, u, ldu, g, ldg,
+                           state, positions, seq_starts, state_slots, width);
     VMX_CHECK_LAUNCH("min_gru");
     return VMX_OK;
 }
