@@ -334,8 +334,15 @@ class VokepelConfig(C.Structure):
     ]
 
 
+# one-family libraries (csrc/Makefile FAMILY=...): the entry points of the other families are absent and stay unbound
+FAMILY_LIBS = ("vokepel",)
+
+
 def _bind():
+    partial = os.environ.get("VMX_LIB_VARIANT") in FAMILY_LIBS
     for name, (res, args) in _SIGS.items():
+        if partial and not hasattr(lib, name):
+            continue
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
         fn.restype = res
         fn.argtypes = args

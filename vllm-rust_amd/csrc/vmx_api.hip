@@ -47,6 +47,10 @@ extern "C" int vmx_init(int device) {
         vmx_set_error("vmx_init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
         return VMX_EUNSUPPORTED;
     }
+#ifdef VMX_FAMILY_BUILD   // a one-family library holds none of the kernels these prepare
+    return VMX_OK;
+#else
     if (int rc = vmx_attention_scratch_init(device)) return rc;
     return vmx_iq_packed_init(device);
+#endif
 }
