@@ -890,10 +890,10 @@ def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16),
     for name in sizes:
         W, H, G, dim, win, R, ff, V, rank = VOKEPEL_SIZES[name]
         sc = 1.0 / math.sqrt(dim)
-        layers = [VokepelLayerSpec(mixer="parallel", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, scale=sc, rot_dims=dim, rot_base=1e6,
-                                   gru_width=R, left_scale=0.6, right_scale=0.5, mlp="dense", ff=ff),
-                  VokepelLayerSpec(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, scale=sc, softcap=50.0, mlp="dense", ff=ff)]
-        spec = VokepelSpec(vocab=V, width=W, layers=layers, residual_mult=0.5, logit_scale=0.5, logit_softcap=15.0, loop=(0, 2, 2))
+        layers = [VokepelLayerSpec(mixer="parallel", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, scale=sc, rot_dims=dim, rot_base=1e4,
+                                   gru_width=R, left_scale=0.5, right_scale=0.5, mlp="dense", ff=ff),
+                  VokepelLayerSpec(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, scale=sc, softcap=30.0, mlp="dense", ff=ff)]
+        spec = VokepelSpec(vocab=V, width=W, layers=layers, residual_mult=0.7, logit_scale=0.8, logit_softcap=30.0, loop=(0, 2, 2))
         model = VokepelForCausalLM(spec, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
         model.load_state(synthetic_weights(spec, 3, device=dev))
         t = _packed_times(model, V, prompt, batches, warmup, steps, side, dev, True)
@@ -913,7 +913,7 @@ def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16),
         if not comparator:
             out[name] = {"vokepel": res}
             continue
-        att = dict(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, keep_first=0, scale=sc, softcap=50.0, mlp="dense", ff=ff)
+        att = dict(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, keep_first=0, scale=sc, softcap=30.0, mlp="dense", ff=ff)
         dlt = dict(mixer="channel_delta", heads=H, kv_heads=H, dim=dim, vdim=dim, conv=4, decay_rank=rank, gate_rank=rank, mlp="dense", ff=ff)
         gs = GupuvikSpec(vocab=V, width=W, layers=[GupuvikLayerSpec(**dlt), GupuvikLayerSpec(**att), GupuvikLayerSpec(**dlt), GupuvikLayerSpec(**att)],
                          embed_scale=1.0)

@@ -497,6 +497,11 @@ def test_greedy_generation_through_the_scheduler(gpu):
     assert all(len(o) == 5 and all(0 <= t < spec.vocab for t in o) for o in outs)
 
 
+def torch_ones(n):
+    import torch
+    return torch.ones(n, dtype=torch.bfloat16)
+
+
 def _write_checkpoint(tmp_path, spec, seed=0):
     from safetensors.torch import save_file
     from vllm_rust_amd.vokepel import synthetic_weights
@@ -504,7 +509,8 @@ def _write_checkpoint(tmp_path, spec, seed=0):
     d = tmp_path / "model"
     d.mkdir()
     (d / "config.json").write_text(json.dumps(spec.to_config()))
-    save_file({k: v.contiguous() for k, v in ck.items()}, str(d / "model.safetensors"))
+    extra = {f"l{i}.norm2": torch_ones(spec.width) for i, l in enumerate(spec.layers) if l.mlp is None}   # a file may carry them: skipped
+    save_file({k: v.contiguous() for k, v in {**ck, **extra}.items()}, str(d / "model.safetensors"))
     return d, {k: v.double() for k, v in ck.items()}
 
 

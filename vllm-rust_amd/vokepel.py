@@ -17,6 +17,7 @@ import ctypes as C
 import dataclasses
 import json
 import math
+import re
 from pathlib import Path
 
 import numpy as np
@@ -59,6 +60,7 @@ class VokepelLayerSpec:
         s.window = int((a.get("mask") or {}).get("size") or 0)
         s.scale = float(a.get("scale", 1.0 / math.sqrt(s.dim)))
         if kind == "attention":
+            s.vdim = s.dim           # the values are the keys
             s.softcap = float(a.get("softcap") or 0.0)
         else:
             rot = a.get("rot") or {}
@@ -261,6 +263,11 @@ class VokepelForCausalLM:
                 dtype = f.info(lib.vmx_safetensors_find(f._h, name.encode()))[1]
                 if dtype != "BF16":
                     raise ValueError(f"{model_dir}: tensor `{name}` is {dtype}; Vokepel checkpoints hold bf16")
+                m = re.fullmatch(r"l(\d+)\.norm2", name)
+                if m and int(m.group(1)) < len(self.spec.layers) and self.spec.layers[int(m.group(1))].mlp is None:
+                    continue                 # the norm of a feed-forward this layer does not have
+                if name in ("loop.in", "loop.step") and not self.spec.loop:
+                    continue                 # the entry of a loop the configuration does not have
                 self.load_tensor(name, ck.get(name))
         finally:
             ck.close()
