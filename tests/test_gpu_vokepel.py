@@ -370,14 +370,20 @@ def test_small_windows_on_page_sizes(gpu, dtype, window, bs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sharp_attention_over_300_tokens_and_long_decoding(gpu, dtype):
+@pytest.mark.parametrize("sizes", ["any", "eights"])
+def test_sharp_attention_over_300_tokens_and_long_decoding(gpu, dtype, sizes):
     """Scores scaled up so that single keys decide rows, windows of 70 / 130 keys over page borders, 220 tokens as a prompt and
     80 decoded one by one; the state of the recurrent unit is carried through all of them."""
     def sharpen(ck):
         for k in ck:
             if k.endswith("mix.q") or k.endswith("left.q"):
                 ck[k] = (ck[k].float() * 3).to(ck[k].dtype)
-    spec = small_spec(layers=[pair_layer(window=70), talk_layer(window=130, scale=1.5), pair_layer(window=0, mlp=None)], loop=(0, 2, 2))
+    if sizes == "any":
+        layers = [pair_layer(window=70), talk_layer(window=130, scale=1.5), pair_layer(window=0, mlp=None)]
+    else:    # multiples of 8: the matrix-core forms in bfloat16, windows over several key tiles
+        layers = [pair_layer(window=70, dim=16, vdim=24, rot_dims=8), talk_layer(window=130, scale=1.5, dim=16),
+                  pair_layer(window=0, mlp=None, dim=32, vdim=8, rot_dims=32)]
+    spec = small_spec(layers=layers, loop=(0, 2, 2))
     model, eng, w = build(spec, dtype, tweak=sharpen, block_size=16, num_blocks=64, max_tokens=512)
     toks = tokens_for(spec, 300, 9)
     want, _ = oracle(spec, w, toks)
