@@ -1197,6 +1197,106 @@ int vmx_vokepel_forward(vmx_vokepel *m, const int32_t *tokens, const int32_t *po
                         const int32_t *state_slots, const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids,
                         float *layer_trace, void *stream);
 
+/* ------------------------------------------------- norm after the sum, head-wise q/k preparation, matrix memories, Gezozen executor */
+
+/* vmx_topk_softmax's selection over sigmoid scores: every expert's f32 logit goes through the logistic function by itself (no
+ * sum over the experts); k rounds of argmax (ties -> smaller index); weights = the chosen scores (renormalize: / their sum). */
+int vmx_topk_sigmoid(const float *logits, float *topk_weights, int32_t *topk_ids, int tokens, int num_experts, int k, int renormalize,
+                     void *stream);
+
+/* What vmx_qk_prepare_ex does differently from vmx_qk_prepare_cache_write. */
+typedef struct vmx_qk_prepare_opts {
+    int norm_per_head;    /* the norms run over each head of head_dim numbers; the gains hold head_dim numbers, the same for every head */
+    int rot_halves;       /* coordinate i turns with i + rot_dims / 2 (i < rot_dims / 2) instead of 2i with 2i + 1 */
+    float rot_mul;        /* cos and sin are multiplied by this (0: 1) */
+    float q_mul, k_mul;   /* constant multipliers of the prepared queries / keys, after the rotation (0: 1) */
+    float *k_out;         /* not NULL: the prepared keys go to these f32 rows (stride ldk_out) and nothing is cached (v, slots, caches unused) */
+    int64_t ldk_out;
+} vmx_qk_prepare_opts;
+/* vmx_qk_prepare_cache_write head by head, with these options; the norms (optional) are per head. */
+int vmx_qk_prepare_ex(float *q_out, const float *q, int64_t ldq, int q_width, const float *k, int64_t ldk, int k_width, const float *v,
+                      int64_t ldv, int v_width, const uint16_t *q_norm_bf16, const uint16_t *k_norm_bf16, float eps, const float *inv_freq,
+                      int rot_dims, int head_dim, const int32_t *positions, const int32_t *slots, void *k_cache, void *v_cache,
+                      int cache_dtype, int tokens, const vmx_qk_prepare_opts *opts, void *stream);
+
+/* vmx_gated_delta_rule's kernel with its options open: g holds a decay per key channel (rows of heads * dim) or, g_per_head, one
+ * per head (rows of heads; ldg 0: one row of constants for every token); beta NULL: the write is the plain outer product
+ * (S <- diag(g_t) S + k_t v_t^T;  o_t = S^T q_t: gated linear attention, retention); the queries are read times q_mul.  State as
+ * vmx_gated_delta_rule_state_bytes. */
+int vmx_matrix_memory_recurrence(float *o, int64_t ldo, const float *q, int64_t ldq, float q_mul, const float *k, int64_t ldk, const float *v,
+                                 int64_t ldv, const float *g, int64_t ldg, int g_per_head, const float *beta, int64_t ldbeta, float *state,
+                                 const int32_t *positions, const int32_t *seq_starts, const int32_t *state_slots, int num_seqs, int heads,
+                                 int qk_heads, int dim, int vdim, void *stream);
+/* In place: g[t, c] <- sigmoid(g[t, c])^(1 / tau) for c < n (through the logarithm). */
+int vmx_sigmoid_root_decay(float *g, int64_t ldg, int tokens, int n, float tau, void *stream);
+/* vmx_head_rms_gate with a SiLU gate (gate_silu: y *= gate * sigmoid(gate)) and an optional gain (w_bf16 NULL: none). */
+int vmx_head_rms_gate_ex(void *y, int y_dtype, const float *o, int64_t ldo, const uint16_t *w_bf16, const float *gate, int64_t ldgate,
+                         int gate_silu, float eps, int tokens, int heads, int vdim, void *stream);
+
+/* A rotary position code: pair i of the first `dims` coordinates of a head turns by position * base^(-2 i / dims).  factor > 0
+ * stretches it for contexts longer than `original` positions: with idx(t) = dims ln(original / (2 pi t)) / (2 ln base),
+ * lo = max(floor(idx(fast)), 0), hi = min(ceil(idx(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair
+ * i turns by step_i (1 - ramp_i) + step_i ramp_i / factor, and cos and sin are multiplied by 0.1 ln(factor) + 1. */
+typedef struct vmx_rotation {
+    int dims;
+    double base;
+    double factor, original, fast, slow;   /* factor 0: plain rotation */
+} vmx_rotation;
+/* The angle steps (f32 [dims / 2], rounded once from double) and the cos / sin multiplier of a rotation. */
+int vmx_rotation_steps(const vmx_rotation *rot, float *steps, float *mul);
+
+#define VMX_MIXER_ATTENTION_GLA 5        /* soft-capped causal attention beside gated linear attention */
+#define VMX_MIXER_ATTENTION_RETENTION 6  /* biased sliding-window attention beside retention */
+#define VMX_MIXER_HEAD_DELTA 7           /* short convolutions + gated delta rule with one decay per head */
+#define VMX_MLP_SIGMOID_MOE 5            /* sigmoid-routed GLU experts (the weight scales the expert's input) + gated shared expert */
+
+/* One layer of a Gezozen model: x <- N1(alpha x + sigmoid(R1 x + r1) * mixer(x)); x <- N2(alpha x + sigmoid(R2 x + r2) * ff(x)). */
+typedef struct vmx_gezozen_layer_config {
+    int mixer;                  /* VMX_MIXER_ATTENTION_GLA, VMX_MIXER_ATTENTION_RETENTION or VMX_MIXER_HEAD_DELTA */
+    /* the attention (left side of the two-sided mixers); for the delta mixer: value heads, query/key heads, key size, value size */
+    int heads, kv_heads, dim, vdim;
+    int window;                 /* 0: every earlier key */
+    float scale, softcap;       /* score scale; soft cap (0: none) */
+    int qkv_bias;               /* q, k and v have biases */
+    vmx_rotation rot;           /* rotation of q and k, in halves (dims 0: none) */
+    /* the recurrent right side */
+    int r_heads, r_dim, r_vdim;
+    float tau;                  /* gated linear attention: decay = sigmoid(z)^(1 / tau) */
+    int decay_rank;             /* gated linear attention: inner size of the decay's two-step projection */
+    const float *decay;         /* retention: host array of r_heads decays (read during create) */
+    vmx_rotation r_rot;         /* retention: rotation of q and k, in halves */
+    float left_scale, right_scale;
+    int conv_taps;              /* delta: taps of the short convolutions */
+    int mlp;                    /* VMX_MLP_NONE or VMX_MLP_SIGMOID_MOE */
+    int experts, top, expert_ff, shared_ff;   /* shared_ff 0: no shared expert */
+} vmx_gezozen_layer_config;
+
+typedef struct vmx_gezozen_config {
+    int vocab, width, num_layers;
+    float norm_eps;
+    int norm_groups;            /* the norms run over this many equal consecutive parts of the row */
+    float postln_alpha;
+    int dtype;                  /* VMX_BF16: bf16 operands and cache; VMX_F32: everything in f32 */
+    int block_size, num_blocks; /* paged key/value cache: rows per block, blocks per layer */
+    int max_tokens, max_seqs;   /* most tokens / sequences of one forward call */
+    int state_slots;            /* recurrent-state slots (one per live sequence) */
+} vmx_gezozen_config;
+
+typedef struct vmx_gezozen vmx_gezozen;
+int vmx_gezozen_create(const vmx_gezozen_config *cfg, const vmx_gezozen_layer_config *layers, vmx_gezozen **out);
+void vmx_gezozen_destroy(vmx_gezozen *m);
+/* One checkpoint tensor under its name in the file: "embed", "head", "final.norm", "l<i>.norm1|norm2", "l<i>.rg1|rg2" (+ ".b"),
+ * two-sided mixers "l<i>.mix.left.q|k|v" (+ ".b"), "mix.left.q.norm|k.norm|o", "l<i>.mix.right.q|k|v|g|o", "mix.right.norm|a1|a2|a2.b";
+ * delta "l<i>.mix.q|k|v" (+ ".conv"), "mix.b|a|A_log|dt_bias|norm|g|o"; "l<i>.mlp.router", "l<i>.mlp.e<j>.gate|up|down",
+ * "l<i>.mlp.shared.gate|up|down|sg": bf16, matrices [out, in]; host or device memory. */
+int vmx_gezozen_load_tensor(vmx_gezozen *m, const char *name, const void *data, size_t bytes, void *stream);
+int vmx_gezozen_missing_tensors(const vmx_gezozen *m);
+/* One step over packed tokens, arguments as vmx_gupuvik_forward. */
+int vmx_gezozen_forward(vmx_gezozen *m, const int32_t *tokens, const int32_t *positions, const int32_t *slots, const int32_t *seq_ids,
+                        int num_tokens, const int32_t *block_tables, int num_seqs, int max_blocks_per_seq, const int32_t *seq_starts,
+                        const int32_t *state_slots, const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids,
+                        float *layer_trace, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -246,6 +246,17 @@ _SIGS = {
     "vmx_vokepel_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
     "vmx_vokepel_missing_tensors": (_i, [_p]),
     "vmx_vokepel_forward": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _p, _p, _i, _p, _p, _p, _p]),
+    "vmx_topk_sigmoid": (_i, [_p, _p, _p, _i, _i, _i, _i, _p]),
+    "vmx_rotation_steps": (_i, [_p, _p, _p]),
+    "vmx_qk_prepare_ex": (_i, [_p, _p, _i64, _i, _p, _i64, _i, _p, _i64, _i, _p, _p, _f, _p, _i, _i, _p, _p, _p, _p, _i, _i, _p, _p]),
+    "vmx_matrix_memory_recurrence": (_i, [_p, _i64, _p, _i64, _f, _p, _i64, _p, _i64, _p, _i64, _i, _p, _i64, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "vmx_sigmoid_root_decay": (_i, [_p, _i64, _i, _i, _f, _p]),
+    "vmx_head_rms_gate_ex": (_i, [_p, _i, _p, _i64, _p, _p, _i64, _i, _f, _i, _i, _i, _p]),
+    "vmx_gezozen_create": (_i, [_p, _p, _p]),
+    "vmx_gezozen_destroy": (None, [_p]),
+    "vmx_gezozen_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
+    "vmx_gezozen_missing_tensors": (_i, [_p]),
+    "vmx_gezozen_forward": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _p, _p, _i, _p, _p, _p, _p]),
 }
 
 
@@ -334,8 +345,36 @@ class VokepelConfig(C.Structure):
     ]
 
 
+class Rotation(C.Structure):
+    """struct vmx_rotation (include/vmx.h)."""
+    _fields_ = [("dims", _i), ("base", C.c_double), ("factor", C.c_double), ("original", C.c_double), ("fast", C.c_double), ("slow", C.c_double)]
+
+
+class QkPrepareOpts(C.Structure):
+    """struct vmx_qk_prepare_opts (include/vmx.h)."""
+    _fields_ = [("norm_per_head", _i), ("rot_halves", _i), ("rot_mul", _f), ("q_mul", _f), ("k_mul", _f), ("k_out", _p), ("ldk_out", _i64)]
+
+
+class GezozenLayerConfig(C.Structure):
+    """struct vmx_gezozen_layer_config (include/vmx.h)."""
+    _fields_ = [
+        ("mixer", _i), ("heads", _i), ("kv_heads", _i), ("dim", _i), ("vdim", _i), ("window", _i), ("scale", _f), ("softcap", _f),
+        ("qkv_bias", _i), ("rot", Rotation), ("r_heads", _i), ("r_dim", _i), ("r_vdim", _i), ("tau", _f), ("decay_rank", _i),
+        ("decay", C.POINTER(_f)), ("r_rot", Rotation), ("left_scale", _f), ("right_scale", _f), ("conv_taps", _i), ("mlp", _i),
+        ("experts", _i), ("top", _i), ("expert_ff", _i), ("shared_ff", _i),
+    ]
+
+
+class GezozenConfig(C.Structure):
+    """struct vmx_gezozen_config (include/vmx.h)."""
+    _fields_ = [
+        ("vocab", _i), ("width", _i), ("num_layers", _i), ("norm_eps", _f), ("norm_groups", _i), ("postln_alpha", _f), ("dtype", _i),
+        ("block_size", _i), ("num_blocks", _i), ("max_tokens", _i), ("max_seqs", _i), ("state_slots", _i),
+    ]
+
+
 # one-family libraries (csrc/Makefile FAMILY=...): the entry points of the other families are absent and stay unbound
-FAMILY_LIBS = ("vokepel",)
+FAMILY_LIBS = ("vokepel", "gezozen")
 
 
 def _bind():

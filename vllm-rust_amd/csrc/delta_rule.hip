@@ -1,5 +1,6 @@
-// Gated delta rule with one decay per key channel, as a recurrent token mixer over packed steps, and the short causal
-// convolution in front of it.  Both carry state from step to step in a SLOT per sequence (the caller's state-slot manager hands
+// Linear recurrences over a matrix memory per head, as recurrent token mixers over packed steps (the gated delta rule with one
+// decay per key channel or per head; the plain decayed outer-product memory of gated linear attention and retention), and the
+// short causal convolution in front of the delta rule.  Both carry state from step to step in a SLOT per sequence (the caller's state-slot manager hands
 // them out); a sequence whose step starts at position 0 starts from zeros whatever its slot held before.
 //
 // Short convolution (vmx_short_conv_silu): y[t, c] = silu(sum_s taps[c, n - 1 - s] * x[t - s, c]), zeros before the sequence's
@@ -9,7 +10,9 @@
 //
 // Recurrence (vmx_gated_delta_rule), per head with a matrix memory S [dim, vdim] in f32:
 //   S <- diag(g_t) S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
-// so a token reads the memory after its own write (computed as (g S)^T q + u (k . q), the same sum in another order).  Query/key
+// so a token reads the memory after its own write (computed as (g S)^T q + u (k . q), the same sum in another order).  The decay
+// g_t is a number per key channel, or one per head (per token, or a constant of the head: row stride 0); without beta the write
+// is the plain outer product, u = v_t (S <- diag(g_t) S + k_t v_t^T: gated linear attention, retention).  Query/key
 // head of value head h: h / (heads / qk_heads).  A workgroup owns 16 value columns of one (sequence, head) and walks the
 // sequence's tokens of the step in order; 16 threads share a column, each holding every 16th row of S in registers, and the
 // column sums per token are 16-lane butterflies.  The state slot keeps S in the workgroup's own register order (the layout is
@@ -116,6 +119,12 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(float *__restrict__ g,
     if (c < heads) beta[(int64_t)t * ldbeta + c] = sigmoid_f(beta[(int64_t)t * ldbeta + c]);
 }
 
+// g[t, c] <- sigmoid(g[t, c])^(1 / tau) in place, through the logarithm: exp(-softplus(-z) / tau)
+__global__ __launch_bounds__(256) void sigmoid_root_decay_kernel(float *__restrict__ g, int64_t ldg, int n, float inv_tau) {
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) g[(int64_t)t * ldg + c] = expf(-softplus_f(-g[(int64_t)t * ldg + c]) * inv_tau);
+}
+
 struct DeltaArgs {
     const float *q, *k, *v, *g, *beta;       // rows of the step: q, k [qk_heads * dim], v [heads * vdim], g [heads * dim], beta [heads]
     int64_t ldq, ldk, ldv, ldg, ldbeta;
@@ -124,6 +133,9 @@ struct DeltaArgs {
     float *state;                            // [slots, heads, tiles, DPT, 256]
     const int32_t *positions, *seq_starts, *state_slots;
     int heads, qk_heads, dim, vdim;
+    int g_per_head;                          // g rows hold one decay per head (ldg 0: the same row for every token) instead of heads * dim
+    int plain;                               // no beta: u = v
+    float q_mul;                             // the queries are multiplied by this constant as they are read
 };
 
 constexpr int DR_RS = 16, DR_VT = 16;   // row splits per column, columns per workgroup
@@ -160,16 +172,16 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const DeltaArgs a
             const int i = tid + 256 * j, tt = i / DP, d = i % DP;
             const int64_t row = first + t0 + tt;
             const bool in = tt < ct && d < a.dim;
-            rq[j] = in ? a.q[row * a.ldq + (int64_t)qh * a.dim + d] : 0.f;
+            rq[j] = in ? a.q[row * a.ldq + (int64_t)qh * a.dim + d] * a.q_mul : 0.f;
             rk[j] = in ? a.k[row * a.ldk + (int64_t)qh * a.dim + d] : 0.f;
-            rg[j] = in ? a.g[row * a.ldg + (int64_t)h * a.dim + d] : 1.f;
+            rg[j] = in ? a.g[row * a.ldg + (a.g_per_head ? (int64_t)h : (int64_t)h * a.dim + d)] : 1.f;
         }
 #pragma unroll
         for (int j = 0; j < NV; j++) {
             const int i = tid + 256 * j, tt = i / DR_VT, cc = tile * DR_VT + i % DR_VT;
             rv[j] = (tt < ct && cc < a.vdim) ? a.v[(int64_t)(first + t0 + tt) * a.ldv + (int64_t)h * a.vdim + cc] : 0.f;
         }
-        rb = tid < ct ? a.beta[(int64_t)(first + t0 + tid) * a.ldbeta + h] : 0.f;
+        rb = (tid < ct && !a.plain) ? a.beta[(int64_t)(first + t0 + tid) * a.ldbeta + h] : 0.f;
     };
     auto stage = [&](int b) {
 #pragma unroll
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const DeltaArgs a
             pk += vmx_dpp<VMX_DPP_XOR2>(pk), pq += vmx_dpp<VMX_DPP_XOR2>(pq), kq += vmx_dpp<VMX_DPP_XOR2>(kq);
             pk += vmx_dpp<VMX_DPP_HALF_MIRROR>(pk), pq += vmx_dpp<VMX_DPP_HALF_MIRROR>(pq), kq += vmx_dpp<VMX_DPP_HALF_MIRROR>(kq);
             pk += vmx_dpp<VMX_DPP_ROR8>(pk), pq += vmx_dpp<VMX_DPP_ROR8>(pq), kq += vmx_dpp<VMX_DPP_ROR8>(kq);
-            const float uu = bv * (vv - pk);
+            const float uu = a.plain ? vv : bv * (vv - pk);
             if (r == 0 && c < a.vdim) a.o[(int64_t)(first + t0 + tt) * a.ldo + (int64_t)h * a.vdim + c] = fmaf(uu, kq, pq);
 #pragma unroll
             for (int u = 0; u < DPT; u++) S[u] = fmaf(kk[u], uu, S[u]);
@@ -245,10 +257,11 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const DeltaArgs a
     for (int u = 0; u < DPT; u++) sp[(int64_t)u * 256] = S[u];
 }
 
-// y[t, h] = o[t, h] / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h]); one wave per (token, head); w bf16 [vdim] shared by heads
+// y[t, h] = o[t, h] / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h]) (gate_silu: * silu(gate[t, h])); one wave per (token, head);
+// w bf16 [vdim] shared by heads (NULL: no gain)
 __global__ __launch_bounds__(256) void head_rms_gate_kernel(void *__restrict__ y, int y_f32, const float *__restrict__ o, int64_t ldo,
                                                              const uint16_t *__restrict__ w, const float *__restrict__ gate, int64_t ldgate,
-                                                             float eps, int rows, int heads, int vdim) {
+                                                             float eps, int rows, int heads, int vdim, int gate_silu) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (row >= rows) return;
     const int t = row / heads, h = row % heads;
@@ -258,8 +271,12 @@ __global__ __launch_bounds__(256) void head_rms_gate_kernel(void *__restrict__ y
     ss = vmx_wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
     for (int i = lane; i < vdim; i += 64) {
-        float v = src[i] * inv * vmx_bf16_to_f32(w[i]);
-        if (gate) v *= sigmoid_f(gate[(int64_t)t * ldgate + (int64_t)h * vdim + i]);
+        float v = src[i] * inv;
+        if (w) v *= vmx_bf16_to_f32(w[i]);
+        if (gate) {
+            const float z = gate[(int64_t)t * ldgate + (int64_t)h * vdim + i];
+            v *= gate_silu ? silu_f(z) : sigmoid_f(z);
+        }
         const int64_t at = ((int64_t)t * heads + h) * vdim + i;
         if (y_f32) ((float *)y)[at] = v;
         else ((uint16_t *)y)[at] = vmx_f32_to_bf16(v);
@@ -343,12 +360,31 @@ extern "C" int vmx_gated_delta_rule(float *o, int64_t ldo, const float *q, int64
                                     int64_t ldv, const float *g, int64_t ldg, const float *beta, int64_t ldbeta, float *state,
                                     const int32_t *positions, const int32_t *seq_starts, const int32_t *state_slots, int num_seqs, int heads,
                                     int qk_heads, int dim, int vdim, void *stream) {
-    VMX_REQUIRE(o && q && k && v && g && beta && state && positions && seq_starts && state_slots, "gated_delta_rule: null pointer");
-    VMX_REQUIRE(heads >= 1 && qk_heads >= 1 && heads % qk_heads == 0, "gated_delta_rule: %d heads do not share %d query/key heads evenly", heads,
-                qk_heads);
-    VMX_REQUIRE(dim >= 1 && dim <= 256 && vdim >= 1, "gated_delta_rule: key size %d outside 1..256", dim);
+    VMX_REQUIRE(beta, "gated_delta_rule: null pointer");
+    return vmx_matrix_memory_recurrence(o, ldo, q, ldq, 1.0f, k, ldk, v, ldv, g, ldg, 0, beta, ldbeta, state, positions, seq_starts, state_slots, num_seqs,
+                                        heads, qk_heads, dim, vdim, stream);
+}
+
+extern "C" int vmx_sigmoid_root_decay(float *g, int64_t ldg, int tokens, int n, float tau, void *stream) {
+    VMX_REQUIRE(g && n >= 1 && ldg >= n && tau > 0.f, "sigmoid_root_decay: bad arguments");
+    if (tokens <= 0) return VMX_OK;
+    hipLaunchKernelGGL(sigmoid_root_decay_kernel, dim3(tokens, (n + 255) / 256), dim3(256), 0, vmx_stream(stream), g, ldg, n, 1.0f / tau);
+    VMX_CHECK_LAUNCH("sigmoid_root_decay");
+    return VMX_OK;
+}
+
+extern "C" int vmx_matrix_memory_recurrence(float *o, int64_t ldo, const float *q, int64_t ldq, float q_mul, const float *k, int64_t ldk, const float *v,
+                                            int64_t ldv, const float *g, int64_t ldg, int g_per_head, const float *beta, int64_t ldbeta,
+                                            float *state, const int32_t *positions, const int32_t *seq_starts, const int32_t *state_slots,
+                                            int num_seqs, int heads, int qk_heads, int dim, int vdim, void *stream) {
+    VMX_REQUIRE(o && q && k && v && g && state && positions && seq_starts && state_slots, "matrix_memory_recurrence: null pointer");
+    VMX_REQUIRE(heads >= 1 && qk_heads >= 1 && heads % qk_heads == 0, "matrix_memory_recurrence: %d heads do not share %d query/key heads evenly",
+                heads, qk_heads);
+    VMX_REQUIRE(dim >= 1 && dim <= 256 && vdim >= 1, "matrix_memory_recurrence: key size %d outside 1..256", dim);
+    VMX_REQUIRE(ldg >= (g_per_head ? heads : (int64_t)heads * dim) || (g_per_head && ldg == 0), "matrix_memory_recurrence: bad decay row stride");
     if (num_seqs <= 0) return VMX_OK;
-    const DeltaArgs a{q, k, v, g, beta, ldq, ldk, ldv, ldg, ldbeta, o, ldo, state, positions, seq_starts, state_slots, heads, qk_heads, dim, vdim};
+    const DeltaArgs a{q, k, v, g, beta, ldq, ldk, ldv, ldg, ldbeta, o, ldo, state, positions, seq_starts, state_slots, heads, qk_heads, dim, vdim,
+                      g_per_head ? 1 : 0, beta ? 0 : 1, q_mul};
     const dim3 grid((vdim + DR_VT - 1) / DR_VT, heads, num_seqs);
     hipStream_t st = vmx_stream(stream);
     int rc;
@@ -358,17 +394,23 @@ extern "C" int vmx_gated_delta_rule(float *o, int64_t ldo, const float *q, int64
         default: rc = delta_launch<16>(a, grid, st); break;
     }
     if (rc) return rc;
-    VMX_CHECK_LAUNCH("gated_delta_rule");
+    VMX_CHECK_LAUNCH("matrix_memory_recurrence");
     return VMX_OK;
 }
 
 extern "C" int vmx_head_rms_gate(void *y, int y_dtype, const float *o, int64_t ldo, const uint16_t *w_bf16, const float *gate, int64_t ldgate,
                                  float eps, int tokens, int heads, int vdim, void *stream) {
-    VMX_REQUIRE(y && o && w_bf16, "head_rms_gate: null pointer");
+    VMX_REQUIRE(w_bf16, "head_rms_gate: null pointer");
+    return vmx_head_rms_gate_ex(y, y_dtype, o, ldo, w_bf16, gate, ldgate, 0, eps, tokens, heads, vdim, stream);
+}
+
+extern "C" int vmx_head_rms_gate_ex(void *y, int y_dtype, const float *o, int64_t ldo, const uint16_t *w_bf16, const float *gate, int64_t ldgate,
+                                    int gate_silu, float eps, int tokens, int heads, int vdim, void *stream) {
+    VMX_REQUIRE(y && o, "head_rms_gate: null pointer");
     VMX_REQUIRE(y_dtype == VMX_F32 || y_dtype == VMX_BF16, "head_rms_gate: f32 or bf16 output");
     if (tokens <= 0) return VMX_OK;
     hipLaunchKernelGGL(head_rms_gate_kernel, dim3((tokens * heads + 3) / 4), dim3(256), 0, vmx_stream(stream), y, y_dtype == VMX_F32, o, ldo,
-                       w_bf16, gate, ldgate, eps, tokens * heads, heads, vdim);
+                       w_bf16, gate, ldgate, eps, tokens * heads, heads, vdim, gate_silu ? 1 : 0);
     VMX_CHECK_LAUNCH("head_rms_gate");
     return VMX_OK;
 }

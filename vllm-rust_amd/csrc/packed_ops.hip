@@ -52,6 +52,82 @@ __global__ __launch_bounds__(256) void rms_norm_f32in_kernel(void *__restrict__ 
     }
 }
 
+// Norm after the sum, over equal consecutive groups of the row: v = acc[t] (w != NULL: every group divided by its own
+// sqrt(mean(group^2) + eps), then times w); x[t] = v (f32), h[t] = v (f32 or bf16: what the next products read), acc[t] = alpha * v
+// (the sum the next sublayer's result is added to).  One workgroup per row, one group after the other.
+__global__ __launch_bounds__(256) void group_norm_post_kernel(float *__restrict__ acc, float *__restrict__ x, void *__restrict__ h, int h_f32,
+                                                               const uint16_t *__restrict__ w, int groups, int width, float eps, float alpha) {
+    __shared__ float red[4];
+    const int64_t row = (int64_t)blockIdx.x * width;
+    const int n = width / groups;
+    for (int g = 0; g < groups; g++) {
+        float inv = 1.0f;
+        if (w) {
+            float ss = 0.f;
+            for (int i = threadIdx.x; i < n; i += 256) {
+                const float v = acc[row + g * n + i];
+                ss = fmaf(v, v, ss);
+            }
+            ss = vmx_block_sum_256(ss, red);
+            inv = 1.0f / sqrtf(ss / (float)n + eps);
+        }
+        for (int i = threadIdx.x; i < n; i += 256) {   // a thread rewrites only what it read itself
+            const int c = g * n + i;
+            float v = acc[row + c] * inv;
+            if (w) v *= vmx_bf16_to_f32(w[c]);
+            x[row + c] = v;
+            if (h_f32) ((float *)h)[row + c] = v;
+            else ((uint16_t *)h)[row + c] = vmx_f32_to_bf16(v);
+            acc[row + c] = alpha * v;
+        }
+    }
+}
+
+// out[r] = x[rows ? rows[r] : r] normed in groups as above, f32 or bf16 (the rows the output matrix reads)
+__global__ __launch_bounds__(256) void group_norm_rows_kernel(void *__restrict__ out, int out_f32, const float *__restrict__ x,
+                                                               const int32_t *__restrict__ rows, const uint16_t *__restrict__ w, int groups,
+                                                               int width, float eps) {
+    __shared__ float red[4];
+    const float *src = x + (int64_t)(rows ? rows[blockIdx.x] : blockIdx.x) * width;
+    const int64_t row = (int64_t)blockIdx.x * width;
+    const int n = width / groups;
+    for (int g = 0; g < groups; g++) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(src[g * n + i], src[g * n + i], ss);
+        ss = vmx_block_sum_256(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+        for (int i = threadIdx.x; i < n; i += 256) {
+            const int c = g * n + i;
+            const float v = src[c] * inv * vmx_bf16_to_f32(w[c]);
+            if (out_f32) ((float *)out)[row + c] = v;
+            else ((uint16_t *)out)[row + c] = vmx_f32_to_bf16(v);
+        }
+    }
+}
+
+// act[r, j] = silu(s g) * (s u) * sigmoid(out_gate[r]) with g = gu[r, j], u = gu[r, up_off + j]: the gated activation of an expert
+// whose INPUT was scaled by s (both products are linear in their input, so the scale is applied to their results), and a
+// sigmoid gate per row on what goes into the down projection (linear too).  s = in_w[in_ids ? in_ids[r] : r] (ids outside
+// [0, in_limit) are padding rows: 0); in_w NULL: 1; out_gate NULL: none.
+__global__ __launch_bounds__(256) void glu_silu_scaled_kernel(void *__restrict__ act, int act_f32, const float *__restrict__ gu, int64_t ldgu,
+                                                               int up_off, int ff, const float *__restrict__ in_w,
+                                                               const int32_t *__restrict__ in_ids, int in_limit,
+                                                               const float *__restrict__ out_gate, int64_t ldgate) {
+    const int64_t r = blockIdx.x;
+    const int j = blockIdx.y * 256 + threadIdx.x;
+    if (j >= ff) return;
+    float s = 1.0f;
+    if (in_w) {
+        const int id = in_ids ? in_ids[r] : (int)r;
+        s = (id >= 0 && id < in_limit) ? in_w[id] : 0.f;
+    }
+    const float g = s * gu[r * ldgu + j], u = s * gu[r * ldgu + up_off + j];
+    float v = g / (1.0f + expf(-g)) * u;
+    if (out_gate) v *= 1.0f / (1.0f + expf(-out_gate[r * ldgate]));
+    if (act_f32) ((float *)act)[r * ff + j] = v;
+    else ((uint16_t *)act)[r * ff + j] = vmx_f32_to_bf16(v);
+}
+
 // inv[pair] = position of the pair in the expert-sorted list
 __global__ __launch_bounds__(256) void moe_inverse_kernel(int32_t *__restrict__ inv, const int32_t *__restrict__ sorted,
                                                            const int32_t *__restrict__ total, int numel) {
@@ -62,7 +138,7 @@ __global__ __launch_bounds__(256) void moe_inverse_kernel(int32_t *__restrict__ 
     }
 }
 
-// x[t] += (sum_slot w[t, slot] * y[inv[t * k + slot]] (slot order) + shared[t]) * sigmoid(gate[t])   (shared, gate optional)
+// x[t] += (sum_slot w[t, slot] * y[inv[t * k + slot]] (slot order) + shared[t]) * sigmoid(gate[t])   (shared, gate optional; w NULL: 1)
 __global__ __launch_bounds__(256) void moe_combine_f32_kernel(float *__restrict__ x, const float *__restrict__ y,
                                                                const int32_t *__restrict__ inv, const float *__restrict__ w, int k,
                                                                const float *__restrict__ shared, const float *__restrict__ gate,
@@ -70,7 +146,7 @@ __global__ __launch_bounds__(256) void moe_combine_f32_kernel(float *__restrict_
     const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;   // tokens on x (no 65535 limit)
     if (i >= width) return;
     float acc = 0.f;
-    for (int s = 0; s < k; s++) acc = fmaf(w[(int64_t)t * k + s], y[(int64_t)inv[(int64_t)t * k + s] * width + i], acc);
+    for (int s = 0; s < k; s++) acc = fmaf(w ? w[(int64_t)t * k + s] : 1.0f, y[(int64_t)inv[(int64_t)t * k + s] * width + i], acc);
     if (shared) acc += shared[(int64_t)t * width + i];
     if (gate) acc *= 1.0f / (1.0f + expf(-gate[(int64_t)t * ldgate + i]));
     x[(int64_t)t * width + i] += acc;
@@ -180,6 +256,33 @@ int vmx_rms_norm_f32in(void *out, int out_f32, const float *x, const int32_t *ro
     if (n <= 0) return VMX_OK;
     hipLaunchKernelGGL(rms_norm_f32in_kernel, dim3(n), dim3(256), 0, st, out, out_f32, x, rows, w, w_scalar, width, eps);
     VMX_CHECK_LAUNCH("rms norm");
+    return VMX_OK;
+}
+
+int vmx_group_norm_post(float *acc, float *x, void *h, int h_f32, const uint16_t *w, int groups, int width, float eps, float alpha, int n,
+                        hipStream_t st) {
+    VMX_REQUIRE(acc && x && h && groups >= 1 && width % groups == 0, "group norm: %d groups do not divide a row of %d", groups, width);
+    if (n <= 0) return VMX_OK;
+    hipLaunchKernelGGL(group_norm_post_kernel, dim3(n), dim3(256), 0, st, acc, x, h, h_f32, w, groups, width, eps, alpha);
+    VMX_CHECK_LAUNCH("group norm");
+    return VMX_OK;
+}
+
+int vmx_group_norm_rows(void *out, int out_f32, const float *x, const int32_t *rows, const uint16_t *w, int groups, int width, float eps, int n,
+                        hipStream_t st) {
+    VMX_REQUIRE(out && x && w && groups >= 1 && width % groups == 0, "group norm: %d groups do not divide a row of %d", groups, width);
+    if (n <= 0) return VMX_OK;
+    hipLaunchKernelGGL(group_norm_rows_kernel, dim3(n), dim3(256), 0, st, out, out_f32, x, rows, w, groups, width, eps);
+    VMX_CHECK_LAUNCH("group norm rows");
+    return VMX_OK;
+}
+
+int vmx_glu_silu_rows_scaled(void *act, int act_f32, const float *gu, int64_t ldgu, int up_off, int rows, int ff, const float *in_w,
+                             const int32_t *in_ids, int in_limit, const float *out_gate, int64_t ldgate, hipStream_t st) {
+    if (rows <= 0) return VMX_OK;
+    hipLaunchKernelGGL(glu_silu_scaled_kernel, dim3(rows, (ff + 255) / 256), dim3(256), 0, st, act, act_f32, gu, ldgu, up_off, ff, in_w, in_ids,
+                       in_limit, out_gate, ldgate);
+    VMX_CHECK_LAUNCH("glu silu (scaled)");
     return VMX_OK;
 }
 

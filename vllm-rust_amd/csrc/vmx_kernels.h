@@ -232,9 +232,20 @@ constexpr int VMX_MOE_FEW_PAIRS = 16;      // most (token, slot) pairs of a step
 int vmx_rms_norm_f32in(void *out, int out_f32, const float *x, const int32_t *rows, const uint16_t *w, int w_scalar, int width, float eps,
                        int n, hipStream_t st);
 int vmx_zero_f32(float *p, int64_t n, hipStream_t st);
+// Norm after the sum over `groups` equal consecutive parts of the row: v = acc[t], each part divided by its own sqrt(mean^2 + eps),
+// times w (w NULL: v = acc[t] as it is); x[t] = v, h[t] = v (f32 or bf16), acc[t] = alpha * v
+int vmx_group_norm_post(float *acc, float *x, void *h, int h_f32, const uint16_t *w, int groups, int width, float eps, float alpha, int n,
+                        hipStream_t st);
+// out[r] = the same norm of x[rows ? rows[r] : r], f32 or bf16
+int vmx_group_norm_rows(void *out, int out_f32, const float *x, const int32_t *rows, const uint16_t *w, int groups, int width, float eps, int n,
+                        hipStream_t st);
+// act[r, j] = silu(s g) (s u) sigmoid(out_gate[r * ldgate]), g = gu[r * ldgu + j], u = gu[r * ldgu + up_off + j],
+// s = in_w[in_ids ? in_ids[r] : r] (ids outside [0, in_limit): 0; in_w NULL: 1); out_gate NULL: no gate
+int vmx_glu_silu_rows_scaled(void *act, int act_f32, const float *gu, int64_t ldgu, int up_off, int rows, int ff, const float *in_w,
+                             const int32_t *in_ids, int in_limit, const float *out_gate, int64_t ldgate, hipStream_t st);
 // inv[pair] = place of the pair in the expert-sorted list (vmx_moe_align_block_size)
 int vmx_moe_inverse(int32_t *inv, const int32_t *sorted, const int32_t *total, int numel, int cap, hipStream_t st);
-// x[t] += (sum_slot w[t, slot] * y[inv[t k + slot]] + shared[t]) * sigmoid(gate[t * ldgate ..]); shared and gate may be NULL
+// x[t] += (sum_slot w[t, slot] * y[inv[t k + slot]] + shared[t]) * sigmoid(gate[t * ldgate ..]); shared and gate may be NULL, w NULL: 1
 int vmx_moe_combine_f32(float *x, const float *y, const int32_t *inv, const float *w, int k, const float *shared, const float *gate,
                         int64_t ldgate, int T, int width, hipStream_t st);
 int vmx_argmax_f32_rows(int32_t *out, unsigned long long *keys, const float *logits, int rows, int vocab, hipStream_t st);

@@ -7,7 +7,10 @@
 // Extras (vmx_window_attention_ex), each optional: a learned sink per head in the softmax denominator (exp(sink), no key, no value);
 // a logarithmic distance penalty s_j -= r1[h] * ln(1 + r2[h] * (i - j)) after the soft cap; mixing of the heads' scores,
 // s_h <- sum_g talk[h, g] s_g at every visible key, before the softmax (all heads of a token then run in one workgroup).
-// vmx_qk_prepare_cache_write readies a step's projected rows: whole-row RMS norms of q and k, pair rotation, cache write.
+// vmx_qk_prepare_cache_write readies a step's projected rows: whole-row RMS norms of q and k, pair rotation, cache write;
+// vmx_qk_prepare_ex does the same head by head (norms over each head with gains shared by the heads, rotation of neighbouring
+// coordinates or of the two halves of the rotated run, scaled cos / sin, constant multipliers, keys to plain rows for a mixer
+// that keeps no cache).
 //
 // Keys and values live in two caches of rows [kv_heads * dim] / [kv_heads * vdim], bf16 or f32; a step writes its new rows first
 // (vmx_kv_cache_write_f32) and prompts, prompt portions and decode tokens then run the SAME kernel over the cache, so a row's
@@ -134,6 +137,80 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(float *__restrict__ q_o
             if (f32) ((float *)vc)[slot * vw + i] = vr[i];
             else ((uint16_t *)vc)[slot * vw + i] = vmx_f32_to_bf16(vr[i]);
         }
+}
+
+struct QkPrep {
+    float *q_out;
+    const float *q, *k, *v;
+    int64_t ldq, ldk, ldv;
+    int qw, kw, vw;
+    const uint16_t *qn, *kn;
+    float eps;
+    const float *inv_freq;
+    int rot_dims, head_dim;
+    const int32_t *positions, *slots;
+    void *kc, *vc;
+    int f32, rot_halves;
+    float rot_mul, q_mul, k_mul;
+    float *k_out;
+    int64_t ldk_out;
+};
+
+// One wave per (token, query or key head): optional RMS norm over the head (gains of head_dim numbers, the same for every head),
+// optional rotation of the head's first rot_dims coordinates, a constant multiplier; queries to q_out, keys to the cache row
+// slots[t] or to k_out[t].  The rotation pairs coordinate i with i + rot_dims / 2 (rot_halves) or 2i with 2i + 1; the partner's
+// value is recomputed from the input row, so lanes exchange nothing but the sum of squares.  Workgroups with blockIdx.y == 0 also
+// store the token's value row.
+__global__ __launch_bounds__(256) void qk_prepare_heads_kernel(const QkPrep a) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int hh = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int qh = a.qw / a.head_dim, kh = a.kw / a.head_dim, hd = a.head_dim;
+    const int64_t slot = a.slots ? a.slots[t] : -1;
+    if (hh < qh + kh) {
+        const bool isq = hh < qh;
+        const int h = isq ? hh : hh - qh;
+        const float *src = (isq ? a.q + (int64_t)t * a.ldq : a.k + (int64_t)t * a.ldk) + (int64_t)h * hd;
+        const uint16_t *w = isq ? a.qn : a.kn;
+        float inv = 1.0f;
+        if (w) {
+            float ss = 0.f;
+            for (int c = lane; c < hd; c += 64) ss = fmaf(src[c], src[c], ss);
+            inv = 1.0f / sqrtf(vmx_wave_sum(ss) / (float)hd + a.eps);
+        }
+        const float pos = (float)a.positions[t], mul = isq ? a.q_mul : a.k_mul;
+        const bool rot = a.inv_freq && a.rot_dims > 0;
+        const int half = a.rot_dims >> 1;
+        for (int c = lane; c < hd; c += 64) {
+            float x = src[c] * inv;
+            if (w) x *= vmx_bf16_to_f32(w[c]);
+            if (rot && c < a.rot_dims) {
+                const bool second = a.rot_halves ? c >= half : (c & 1);
+                const int pc = a.rot_halves ? (second ? c - half : c + half) : (c ^ 1);
+                const int fi = a.rot_halves ? (second ? c - half : c) : (c >> 1);
+                float y = src[pc] * inv;
+                if (w) y *= vmx_bf16_to_f32(w[pc]);
+                float sn, cs;
+                sincosf(pos * a.inv_freq[fi], &sn, &cs);
+                sn *= a.rot_mul, cs *= a.rot_mul;
+                x = second ? x * cs + y * sn : x * cs - y * sn;
+            }
+            x *= mul;
+            const int e = h * hd + c;
+            if (isq) a.q_out[(int64_t)t * a.qw + e] = x;
+            else if (a.k_out) a.k_out[(int64_t)t * a.ldk_out + e] = x;
+            else if (slot >= 0) {
+                if (a.f32) ((float *)a.kc)[slot * a.kw + e] = x;
+                else ((uint16_t *)a.kc)[slot * a.kw + e] = vmx_f32_to_bf16(x);
+            }
+        }
+    }
+    if (blockIdx.y == 0 && a.v && a.vc && slot >= 0) {
+        const float *vr = a.v + (int64_t)t * a.ldv;
+        for (int i = threadIdx.x; i < a.vw; i += 256) {
+            if (a.f32) ((float *)a.vc)[slot * a.vw + i] = vr[i];
+            else ((uint16_t *)a.vc)[slot * a.vw + i] = vmx_f32_to_bf16(vr[i]);
+        }
+    }
 }
 
 constexpr int WA_MAX_DIM = 256;
@@ -922,6 +999,36 @@ extern "C" int vmx_qk_prepare_cache_write(float *q_out, const float *q, int64_t 
                        q_norm_bf16, k_norm_bf16, eps, inv_freq, rot ? rot_dims : 0, head_dim, positions, slots, k_cache, v_cache,
                        cache_dtype == VMX_F32);
     VMX_CHECK_LAUNCH("qk_prepare");
+    return VMX_OK;
+}
+
+extern "C" int vmx_qk_prepare_ex(float *q_out, const float *q, int64_t ldq, int q_width, const float *k, int64_t ldk, int k_width, const float *v,
+                                 int64_t ldv, int v_width, const uint16_t *q_norm_bf16, const uint16_t *k_norm_bf16, float eps,
+                                 const float *inv_freq, int rot_dims, int head_dim, const int32_t *positions, const int32_t *slots,
+                                 void *k_cache, void *v_cache, int cache_dtype, int tokens, const vmx_qk_prepare_opts *opts, void *stream) {
+    VMX_REQUIRE(opts, "qk_prepare_ex: null options");
+    const vmx_qk_prepare_opts &o = *opts;
+    const bool cached = o.k_out == nullptr;
+    VMX_REQUIRE(q_out && q && k && positions, "qk_prepare_ex: null pointer");
+    VMX_REQUIRE(!cached || (v && slots && k_cache && v_cache), "qk_prepare_ex: a cache write needs values, slots and both caches");
+    VMX_REQUIRE(cached || o.ldk_out >= k_width, "qk_prepare_ex: bad key row stride");
+    VMX_REQUIRE(q_out != q && o.k_out != k, "qk_prepare_ex: the prepared rows need memory of their own");
+    VMX_REQUIRE(cache_dtype == VMX_F32 || cache_dtype == VMX_BF16, "qk_prepare_ex: the cache holds f32 or bf16");
+    VMX_REQUIRE(q_width >= 1 && k_width >= 1 && ldq >= q_width && ldk >= k_width && (!cached || (v_width >= 1 && ldv >= v_width)),
+                "qk_prepare_ex: bad row widths");
+    VMX_REQUIRE(head_dim >= 1 && q_width % head_dim == 0 && k_width % head_dim == 0, "qk_prepare_ex: rows are not whole heads of %d", head_dim);
+    VMX_REQUIRE(o.norm_per_head || (!q_norm_bf16 && !k_norm_bf16), "qk_prepare_ex: whole-row norms are vmx_qk_prepare_cache_write's");
+    const bool rot = inv_freq && rot_dims > 0;
+    VMX_REQUIRE(!rot || (rot_dims % 2 == 0 && rot_dims <= head_dim && (o.rot_halves || head_dim % 2 == 0)),
+                "qk_prepare_ex: %d rotated coordinates in heads of %d", rot_dims, head_dim);
+    if (tokens <= 0) return VMX_OK;
+    const QkPrep a{q_out, q, k, cached ? v : nullptr, ldq, ldk, ldv, q_width, k_width, v_width, q_norm_bf16, k_norm_bf16, eps, inv_freq,
+                   rot ? rot_dims : 0, head_dim, positions, cached ? slots : nullptr, cached ? k_cache : nullptr, cached ? v_cache : nullptr,
+                   cache_dtype == VMX_F32, o.rot_halves ? 1 : 0, o.rot_mul != 0.f ? o.rot_mul : 1.0f, o.q_mul != 0.f ? o.q_mul : 1.0f,
+                   o.k_mul != 0.f ? o.k_mul : 1.0f, o.k_out, o.ldk_out};
+    const int heads = (q_width + k_width) / head_dim;
+    hipLaunchKernelGGL(qk_prepare_heads_kernel, dim3(tokens, (heads + 3) / 4), dim3(256), 0, vmx_stream(stream), a);
+    VMX_CHECK_LAUNCH("qk_prepare_ex");
     return VMX_OK;
 }
 
