@@ -8,7 +8,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent.parent
 LIB = ROOT / "vllm-rust_amd" / "lib"
 # architectures (config.json) whose kernels build as a library of their own (csrc/Makefile FAMILY=...)
-FAMILY_OF = {"Vokepel": "vokepel"}
+FAMILY_OF = {"Vokepel": "vokepel", "Gezozen": "gezozen"}
 
 
 def _family(model_dir):

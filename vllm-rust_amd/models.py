@@ -55,6 +55,14 @@ def _load_vokepel(model_dir, dtype, max_tokens, max_seqs, block_size, device):
                                               max_seqs=max_seqs, device=device)
 
 
+@register("Gezozen")
+def _load_gezozen(model_dir, dtype, max_tokens, max_seqs, block_size, device):
+    from .gezozen import GezozenForCausalLM
+    return GezozenForCausalLM.from_pretrained(model_dir, dtype=dtype, block_size=block_size,
+                                              num_blocks=_cache_geometry(max_tokens, max_seqs, block_size), max_tokens=max_tokens,
+                                              max_seqs=max_seqs, device=device)
+
+
 @register("Qwen3ForCausalLM")
 def _load_qwen3(model_dir, dtype, max_tokens, max_seqs, block_size, device):
     """AWQ / GPTQ / EXL3 Qwen3 checkpoints (the quantization is detected from the directory)."""
