@@ -940,6 +940,93 @@ def vokepel_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16),
             "prompt": prompt, "sizes": out}
 
 
+GEZOZEN_SIZES = {
+    # name: (width, heads, kv_heads, dim, window, recurrent heads of the two-sided mixers, experts, top, expert_ff, shared_ff, decay rank, vocab)
+    "1k": (1024, 8, 2, 128, 1024, 4, 16, 4, 512, 1024, 64, 32000),
+    "2k": (2048, 16, 4, 128, 4096, 8, 32, 4, 1024, 2048, 128, 32000),
+}
+
+
+def gezozen_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16), comparator=True, main=True):
+    """Gezozen (layers that normalise after the sum: attention beside gated linear attention / beside retention, gated delta rule
+    with one decay per head; sigmoid-routed experts whose score scales their input, a gated shared expert; bf16 weights) at layer
+    sizes of real models, beside the closest existing model at equal size: Gupuvik, the other packed-step executor with window
+    attention, a gated delta rule over state slots, gated residuals and SiLU-gated experts.  Gezozen: delta + experts, attention |
+    gated linear attention + experts, windowed attention | retention + experts, delta + experts; Gupuvik: delta rule + experts,
+    attention + experts, attention + experts, delta rule + experts with the same width, heads, head sizes, window, experts and
+    vocabulary.  Prompt pass: tokens/s of one `prompt`-token sequence; decode: aggregate tok/s of B sequences at context `prompt`,
+    one hipGraph per step.  main=False times the comparator alone (kernel traces of one model)."""
+    from vllm_rust_amd.gezozen import GezozenForCausalLM, GezozenLayerSpec, GezozenSpec, RotationSpec, synthetic_weights
+    from vllm_rust_amd.gupuvik import GupuvikForCausalLM, GupuvikLayerSpec, GupuvikSpec
+    from vllm_rust_amd.gupuvik import synthetic_weights as gupuvik_weights
+    out = {}
+    dev = torch.device("cuda", torch.cuda.current_device())
+    side = torch.cuda.Stream(device=dev)
+    BM = max(batches)
+    per_seq = (prompt + warmup + steps + 8 + 15) // 16 + 1
+    for name in sizes:
+        W, H, G, dim, win, RH, E, top, ff, sff, rank, V = GEZOZEN_SIZES[name]
+        sc = 1.0 / math.sqrt(dim)
+        moe = dict(mlp="moe", experts=E, top=top, expert_ff=ff, shared_ff=sff)
+        two = dict(heads=H, kv_heads=G, dim=dim, vdim=dim, scale=sc, r_heads=RH, r_dim=dim, r_vdim=dim, left_scale=0.5, right_scale=1.0)
+        dlt = GezozenLayerSpec(mixer="delta", heads=H, kv_heads=G, dim=dim, vdim=dim, conv=4, **moe)
+        gla = GezozenLayerSpec(mixer="parallel", softcap=50.0, rot=RotationSpec(dim // 2, 1e4), tau=8.0, decay_rank=rank, **two, **moe)
+        ret = GezozenLayerSpec(mixer="parallel_2", window=win, rot=RotationSpec(dim // 2, 1e5, dict(factor=8.0, original=4096.0, fast=16.0, slow=2.0)),
+                               decay=tuple(1.0 - 2.0 ** (-5 - 5 * i / max(RH - 1, 1)) for i in range(RH)), r_rot=RotationSpec(dim // 2, 1e4), **two, **moe)
+        spec = GezozenSpec(vocab=V, width=W, layers=[dlt, gla, ret, dlt], norm_groups=4, postln_alpha=2.0)
+        t = {"prefill": float("inf"), **{B: float("inf") for B in batches}}
+        if main:
+            model = GezozenForCausalLM(spec, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+            model.load_state(synthetic_weights(spec, 3, device=dev))
+            t = _packed_times(model, V, prompt, batches, warmup, steps, side, dev, True)
+            model.close()
+            del model
+        hd, gd, rd = H * dim, G * dim, RH * dim
+        ffl = W * W + (E + 2 * sff + 1) * W + sff * W + top * 3 * ff * W          # gate 2, router, shared expert, the chosen experts
+        mix_dlt = W * (2 * gd + hd + 2 * H + hd + W) + hd * W
+        mix_gla = W * (hd + 2 * gd + 4 * rd + rank + W) + rank * rd + hd * W + rd * W
+        mix_ret = W * (hd + 2 * gd + 4 * rd + W) + hd * W + rd * W
+        lin = 2 * mix_dlt + mix_gla + mix_ret + 4 * ffl
+        att_fl = H * 2 * dim * (prompt / 2 + min(win, prompt / 2))                # one causal and one windowed attention (MACs per token)
+        rec_fl = (2 * H + 2 * RH) * 3 * dim * dim                                 # decay + two rank-one passes per token and head
+        res = {"prefill": {"tokens": prompt, "ms": round(t["prefill"] * 1e3, 3), "tok_s": round(prompt / t["prefill"], 1),
+                           "TFLOP_s": round(2.0 * prompt * (lin + att_fl + rec_fl + V * W / prompt) / t["prefill"] / 1e12, 2)}}
+        wfixed = 2 * (2 * mix_dlt + mix_gla + mix_ret + 4 * (ffl - top * 3 * ff * W) + V * W)
+        for B in batches:
+            by = wfixed + 2 * 4 * min(E, B * top) * 3 * ff * W + 2 * B * (prompt + 1 + min(win, prompt + 1)) * 2 * gd + 2 * B * (2 * H + 2 * RH) * dim * dim * 4
+            res[f"decode_b{B}"] = {"tok_s": round(B / t[B], 1), "ms_per_step": round(t[B] * 1e3, 4), "GBps_algorithmic": round(by / t[B] / 1e9, 1)}
+        if not comparator:
+            out[name] = {"gezozen": res}
+            continue
+        gmoe = dict(mlp="moe", experts=E, top=top, expert_ff=ff)
+        att = dict(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=dim, window=win, keep_first=0, scale=sc, softcap=30.0)
+        gdl = dict(mixer="channel_delta", heads=H, kv_heads=G, dim=dim, vdim=dim, conv=4, decay_rank=rank, gate_rank=rank)
+        gs = GupuvikSpec(vocab=V, width=W, layers=[GupuvikLayerSpec(**gdl, **gmoe), GupuvikLayerSpec(**dict(att, window=0), **gmoe),
+                                                   GupuvikLayerSpec(**att, **gmoe), GupuvikLayerSpec(**gdl, **gmoe)], embed_scale=1.0)
+        gm = GupuvikForCausalLM(gs, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+        gm.load_state(gupuvik_weights(gs, 3, device=dev))
+        tg = _packed_times(gm, V, prompt, batches, warmup, steps, side, dev, True)
+        gm.close()
+        del gm
+        g_att = W * (hd + 2 * gd + H) + hd * W
+        g_dlt = W * (2 * gd + hd + H + 2 * rank) + rank * 2 * hd + hd * W
+        gffl = (E + top * 3 * ff) * W
+        glin = 2 * (g_att + g_dlt) + 4 * (2 * W * W + gffl)
+        gres = {"prefill": {"tokens": prompt, "ms": round(tg["prefill"] * 1e3, 3), "tok_s": round(prompt / tg["prefill"], 1),
+                            "TFLOP_s": round(2.0 * prompt * (glin + att_fl + 2 * H * 3 * dim * dim + V * W / prompt) / tg["prefill"] / 1e12, 2)}}
+        gfixed = 2 * (2 * (g_att + g_dlt) + 4 * (2 * W * W + E * W) + 2 * V * W)
+        for B in batches:
+            by = gfixed + 2 * 4 * min(E, B * top) * 3 * ff * W + 2 * B * (prompt + 1 + min(win, prompt + 1)) * 2 * gd + 2 * 2 * B * H * dim * dim * 4
+            gres[f"decode_b{B}"] = {"tok_s": round(B / tg[B], 1), "ms_per_step": round(tg[B] * 1e3, 4), "GBps_algorithmic": round(by / tg[B] / 1e9, 1)}
+        out[name] = {**({"gezozen": res} if main else {}), "gupuvik": gres,
+                     "config": {"width": W, "layers": ["delta+moe", "parallel+moe", "parallel_2+moe", "delta+moe"], "heads": H, "kv_heads": G, "dim": dim,
+                                "window": win, "recurrent_heads": RH, "experts": E, "top": top, "expert_ff": ff, "shared_ff": sff, "decay_rank": rank,
+                                "vocab": V, "gupuvik": {"layers": ["channel_delta+moe", "attention+moe", "attention(window)+moe", "channel_delta+moe"],
+                                                        "rank": rank, "conv": 4}}}
+    return {"metric": "Gezozen prompt and decode throughput beside Gupuvik at equal size", "unit": "tok/s", "dtype": "bf16", "data": "synthetic",
+            "prompt": prompt, "sizes": out}
+
+
 def plan_job(gpus, world, replicas_flag, weights, local_ranks):
     """What a launch of this script measures -- pure argument logic, no device.  N = 1: the single-GPU job.  N > 1 (one process
     per GPU under torch.distributed.run): ONE model tensor-parallel over the N ranks (BASELINE.json's metric is the TP curve at
@@ -1096,16 +1183,20 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary measurements (other models at N = 1, replicas at N > 1)")
     ap.add_argument("--no-moe", action="store_true", help="skip the Mixtral-8x7B-shaped fused-MoE secondary measurement")
-    ap.add_argument("--no-comparator", action="store_true", help="--workload vokepel: time the Vokepel executor alone (kernel traces of one model)")
-    ap.add_argument("--sizes", default="1k,2k", help="--workload vokepel: which of its sizes to run")
-    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel"], default="all",
+    ap.add_argument("--no-comparator", action="store_true",
+                    help="--workload vokepel / gezozen: time that executor alone (kernel traces of one model)")
+    ap.add_argument("--comparator-only", action="store_true", help="--workload gezozen: time the comparator alone (kernel traces of one model)")
+    ap.add_argument("--sizes", default="1k,2k", help="--workload vokepel / gezozen: which of its sizes to run")
+    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel", "gezozen"], default="all",
                     help="profiling aid: run ONE workload alone (qwen3 = the primary without secondaries; the others print only "
                          "their own block), so that a kernel trace of the run holds that workload's launches only; gesutar = the Gesutar "
                          "executor (latent attention + grouped-router MoE, bf16) at two layer sizes beside the bf16 dense Qwen3 executor at "
                          "equal size: prompt tok/s and decode tok/s at 1 and 16 sequences (not part of the default run); gupuvik = the Gupuvik "
                          "executor (window attention / gated delta rule, gated residuals, bf16) at two layer sizes beside Gesutar at equal size, "
                          "the same measurements; vokepel = the Vokepel executor (looped pre-norm layers, rotary sink attention beside a minimal "
-                         "gated recurrent unit, mixed-head attention, bf16) at two layer sizes beside Gupuvik at equal size, the same measurements")
+                         "gated recurrent unit, mixed-head attention, bf16) at two layer sizes beside Gupuvik at equal size, the same measurements; "
+                         "gezozen = the Gezozen executor (norm after the sum, attention beside gated linear attention / retention, per-head "
+                         "gated delta rule, sigmoid-routed experts, bf16) at two layer sizes beside Gupuvik at equal size, the same measurements")
     ap.add_argument("--tp", action="store_true", help="accepted for compatibility: with --gpus N > 1 the tensor-parallel job is the default")
     ap.add_argument("--replicas", action="store_true",
                     help="with --gpus N > 1: N independent replicas as the primary (weak scaling, no collective) instead of ONE model "
@@ -1120,8 +1211,11 @@ def main():
     plan = plan_job(args.gpus, world, args.replicas, args.weights, d.local)
 
     K_steps, W_steps = args.steps, args.warmup
-    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel"):   # one secondary alone (single GPU)
-        if args.workload == "vokepel":
+    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar", "gupuvik", "vokepel", "gezozen"):   # one secondary alone (single GPU)
+        if args.workload == "gezozen":
+            blk = gezozen_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup,
+                                   sizes=tuple(args.sizes.split(",")), comparator=not args.no_comparator, main=not args.comparator_only)
+        elif args.workload == "vokepel":
             blk = vokepel_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup,
                                    sizes=tuple(args.sizes.split(",")), comparator=not args.no_comparator)
         elif args.workload == "gupuvik":
